@@ -1,0 +1,40 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+GOLDEN = os.path.join(ROOT, "tests", "golden")
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(scope="session")
+def fixture_ids_mask():
+    """The two data fixtures the reference ships (bloomz-7b/xinput.ids.bin and
+    xinput.mask.bin): int32 little-endian [2, 512]."""
+    ids = np.fromfile(os.path.join(GOLDEN, "xinput.ids.bin"), dtype="<i4").reshape(2, 512)
+    mask = np.fromfile(os.path.join(GOLDEN, "xinput.mask.bin"), dtype="<i4").reshape(2, 512)
+    return ids.astype(np.int32), mask.astype(np.int32)
+
+
+def assert_close(got, ref, rtol, what=""):
+    """|got - ref| <= rtol * (|ref| + rms(ref)) elementwise: a relative bound
+    with a floor tied to the tensor's own scale, so entries that are zero by
+    cancellation do not demand infinite precision."""
+    got = np.asarray(got, np.float64)
+    ref = np.asarray(ref, np.float64)
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    assert np.all(np.isfinite(got)), what + ": non-finite values"
+    rms = float(np.sqrt(np.mean(ref * ref))) if ref.size else 0.0
+    bound = rtol * (np.abs(ref) + rms) + 1e-30
+    err = np.abs(got - ref)
+    worst = float(np.max(err / bound)) if ref.size else 0.0
+    assert worst <= 1.0, "%s: worst error %.3g x the %.1e bound (rms %.3g)" % (
+        what, worst, rtol, rms)
