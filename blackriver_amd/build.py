@@ -1,0 +1,100 @@
+"""Builds the native libraries in-tree.
+
+  libbr_hip.so       HIP kernels + C ABI (hipcc, gfx950 only)
+  libblackriver.so   C++ host runtime: operator API, tensors, word VM
+                     (g++, links libbr_hip.so; never includes a HIP header)
+
+Run as ``python -m blackriver_amd.build``.  hipcc cross-compiles for gfx950
+without a GPU, so this works on a CPU-only machine.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+INCLUDE = os.path.join(ROOT, "include")
+KERNEL_DIR = os.path.join(PKG, "csrc", "kernels")
+HOST_DIR = os.path.join(PKG, "csrc", "host")
+LIB_DIR = os.path.join(PKG, "lib")
+OBJ_DIR = os.path.join(PKG, "build")
+
+HIP_LIB = os.path.join(LIB_DIR, "libbr_hip.so")
+HOST_LIB = os.path.join(LIB_DIR, "libblackriver.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + KERNEL_DIR,
+    # keep the compiler from forming packed-fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-I" + INCLUDE, "-I" + HOST_DIR]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def _sources(folder, ext):
+    return sorted(os.path.join(folder, f) for f in os.listdir(folder) if f.endswith(ext))
+
+
+def build_kernels(verbose=True):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = _sources(KERNEL_DIR, ".hip")
+    objs = [os.path.join(OBJ_DIR, os.path.basename(s)[:-4] + ".o") for s in srcs]
+
+    def one(pair):
+        src, obj = pair
+        return _run(["hipcc"] + HIPCC_FLAGS + ["-c", src, "-o", obj])
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        for out in pool.map(one, zip(srcs, objs)):
+            if verbose and out.strip():
+                print(out)
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB] + objs)
+    if verbose:
+        print("built", HIP_LIB)
+    return HIP_LIB
+
+
+def build_host(verbose=True):
+    srcs = _sources(HOST_DIR, ".cpp") if os.path.isdir(HOST_DIR) else []
+    if not srcs:
+        return None
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [os.path.join(OBJ_DIR, "host_" + os.path.basename(s)[:-4] + ".o") for s in srcs]
+
+    def one(pair):
+        src, obj = pair
+        return _run(["g++"] + CXX_FLAGS + ["-c", src, "-o", obj])
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        for out in pool.map(one, zip(srcs, objs)):
+            if verbose and out.strip():
+                print(out)
+    _run(["g++", "-shared", "-fPIC", "-o", HOST_LIB] + objs +
+         ["-L" + LIB_DIR, "-lbr_hip", "-Wl,-rpath,$ORIGIN"])
+    if verbose:
+        print("built", HOST_LIB)
+    return HOST_LIB
+
+
+def build_all(verbose=True):
+    build_kernels(verbose)
+    build_host(verbose)
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

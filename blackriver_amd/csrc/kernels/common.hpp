@@ -1,0 +1,101 @@
+// Shared device helpers for the gfx950 kernels: wave64 / workgroup reductions,
+// 128-bit vector types and the launch-check macros used by every C-ABI entry.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "br_hip.h"
+
+namespace brk {
+
+constexpr int kWave = 64;  // CDNA wavefront width
+
+// Returns from the enclosing extern "C" function with the hipError_t value.
+#define BR_HIP_TRY(expr)                         \
+    do {                                         \
+        hipError_t br_err_ = (expr);             \
+        if (br_err_ != hipSuccess) return (int)br_err_; \
+    } while (0)
+
+// After a kernel launch: report launch-configuration errors to the caller.
+#define BR_HIP_LAUNCH_CHECK() BR_HIP_TRY(hipGetLastError())
+
+inline hipStream_t as_stream(br_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned8(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; }
+
+// ---- wave64 reductions: butterfly over the 64 lanes --------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Workgroup sum of NV values per thread; every thread gets the result.
+// `lds` must hold NV * (blockDim.x / 64) floats and must not be reused by the
+// caller before the next __syncthreads() it issues itself (callers alternate
+// between two such buffers to get away with one barrier per reduction).
+template <int NV>
+__device__ __forceinline__ void block_sum(float (&v)[NV], float* lds) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int nwave = blockDim.x >> 6;
+#pragma unroll
+    for (int i = 0; i < NV; i++) v[i] = wave_sum(v[i]);
+    if (nwave == 1) return;
+    if (lane == 0) {
+#pragma unroll
+        for (int i = 0; i < NV; i++) lds[i * nwave + wave] = v[i];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        float s = 0.f;
+        for (int w = 0; w < nwave; w++) s += lds[i * nwave + w];
+        v[i] = s;
+    }
+}
+
+// ---- fp16 pack / unpack (8 halves <-> one 128-bit register quad) --------
+struct alignas(16) half8 {
+    __half2 v[4];
+};
+struct alignas(8) half4 {
+    __half2 v[2];
+};
+
+__device__ __forceinline__ void unpack8(const half8& h, float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float2 t = __half22float2(h.v[i]);
+        f[2 * i] = t.x;
+        f[2 * i + 1] = t.y;
+    }
+}
+
+__device__ __forceinline__ half8 pack8(const float (&f)[8]) {
+    half8 h;
+#pragma unroll
+    for (int i = 0; i < 4; i++) h.v[i] = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
+    return h;
+}
+
+// Grid size for a grid-stride elementwise kernel: enough workgroups to keep
+// 256 CUs busy several times over, never more than the work needs.
+inline int grid_for(int64_t work_items, int block, int max_blocks = 256 * 16) {
+    int64_t g = (work_items + block - 1) / block;
+    if (g < 1) g = 1;
+    if (g > max_blocks) g = max_blocks;
+    return (int)g;
+}
+
+}  // namespace brk

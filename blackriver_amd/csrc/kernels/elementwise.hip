@@ -1,0 +1,784 @@
+// Memory-bound elementwise kernels for gfx950: fill, cast, broadcast add,
+// (bias-)GELU forward / backward, transpose 0213, column sums and the
+// data-preparation tables.  All of them move 128 bits per lane per access and
+// are launched as grid-stride loops over a few thousand workgroups.
+#include "common.hpp"
+
+#include <float.h>
+#include <hip/hip_bf16.h>
+
+using namespace brk;
+
+namespace {
+
+constexpr int kBlock = 256;
+
+// ------------------------------------------------------------------ fill
+template <typename T>
+__global__ __launch_bounds__(kBlock) void fill_kernel(T* dst, T value, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) dst[i] = value;
+}
+
+// ------------------------------------------------------------------ cast
+template <typename T>
+__device__ __forceinline__ float to_f32(T v);
+template <>
+__device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ float to_f32<__half>(__half v) { return __half2float(v); }
+template <>
+__device__ __forceinline__ float to_f32<__hip_bfloat16>(__hip_bfloat16 v) { return __bfloat162float(v); }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ __half from_f32<__half>(float v) { return __float2half_rn(v); }
+template <>
+__device__ __forceinline__ __hip_bfloat16 from_f32<__hip_bfloat16>(float v) { return __float2bfloat16(v); }
+
+template <typename S, typename D>
+__global__ __launch_bounds__(kBlock) void cast_kernel(const S* src, D* dst, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock * 4;
+    for (int64_t i = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * 4; i < n; i += stride) {
+        if (i + 3 < n) {
+            S s[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) s[j] = src[i + j];
+#pragma unroll
+            for (int j = 0; j < 4; j++) dst[i + j] = from_f32<D>(to_f32<S>(s[j]));
+        } else {
+            for (int64_t j = i; j < n; j++) dst[j] = from_f32<D>(to_f32<S>(src[j]));
+        }
+    }
+}
+
+template <typename S>
+int cast_from(const void* src, void* dst, int dst_dtype, int64_t n, hipStream_t st) {
+    const int grid = grid_for((n + 3) / 4, kBlock);
+    switch (dst_dtype) {
+        case BR_F32: cast_kernel<S, float><<<grid, kBlock, 0, st>>>((const S*)src, (float*)dst, n); break;
+        case BR_F16: cast_kernel<S, __half><<<grid, kBlock, 0, st>>>((const S*)src, (__half*)dst, n); break;
+        case BR_BF16:
+            cast_kernel<S, __hip_bfloat16><<<grid, kBlock, 0, st>>>((const S*)src, (__hip_bfloat16*)dst, n);
+            break;
+        default: return BR_ERR_TODO;
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+// --------------------------------------------------------- broadcast add
+// Same-shape fast path: 128-bit loads, no index arithmetic.
+__global__ __launch_bounds__(kBlock) void add_same_f32x4(const float4* a, const float4* b, float4* c,
+                                                          int64_t n4) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) {
+        float4 x = a[i], y = b[i];
+        c[i] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void add_same_f16x8(const half8* a, const half8* b, half8* c,
+                                                          int64_t n8) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += stride) {
+        half8 x = a[i], y = b[i], z;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            // add in fp32 and round once, like a + b on fp16 values
+            float2 fx = __half22float2(x.v[j]), fy = __half22float2(y.v[j]);
+            z.v[j] = __floats2half2_rn(fx.x + fy.x, fx.y + fy.y);
+        }
+        c[i] = z;
+    }
+}
+
+struct BcastDims {
+    unsigned s1, s2, s3v;      // a's dims 1,2 and dim 3 in vectors
+    long long bst0, bst1, bst2;  // b's element strides (0 where broadcast)
+    int bst3;                    // 0 when b's last dim is broadcast, else 1
+};
+
+// General path over vectors of 4 fp32 along the last dimension.
+__global__ __launch_bounds__(kBlock) void add_bcast_f32x4(const float* a, const float* b, float* c,
+                                                           long long nvec, BcastDims d) {
+    const long long stride = (long long)gridDim.x * kBlock;
+    for (long long v = (long long)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += stride) {
+        unsigned long long r = (unsigned long long)v;
+        const unsigned i3v = (unsigned)(r % d.s3v);
+        r /= d.s3v;
+        const unsigned i2 = (unsigned)(r % d.s2);
+        r /= d.s2;
+        const unsigned i1 = (unsigned)(r % d.s1);
+        const unsigned long long i0 = r / d.s1;
+        const float4 x = reinterpret_cast<const float4*>(a)[v];
+        const float* bp = b + i0 * d.bst0 + i1 * d.bst1 + i2 * d.bst2;
+        float4 y;
+        if (d.bst3) {
+            y = *reinterpret_cast<const float4*>(bp + (long long)i3v * 4);
+        } else {
+            const float s = bp[0];
+            y = make_float4(s, s, s, s);
+        }
+        reinterpret_cast<float4*>(c)[v] = make_float4(x.x + y.x, x.y + y.y, x.z + y.z, x.w + y.w);
+    }
+}
+
+// Fallback for shapes / pointers that do not allow 128-bit accesses.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void add_bcast_scalar(const T* a, const T* b, T* c, long long n,
+                                                            unsigned s1, unsigned s2, unsigned s3,
+                                                            long long bst0, long long bst1,
+                                                            long long bst2, int bst3) {
+    const long long stride = (long long)gridDim.x * kBlock;
+    for (long long v = (long long)blockIdx.x * kBlock + threadIdx.x; v < n; v += stride) {
+        unsigned long long r = (unsigned long long)v;
+        const unsigned i3 = (unsigned)(r % s3);
+        r /= s3;
+        const unsigned i2 = (unsigned)(r % s2);
+        r /= s2;
+        const unsigned i1 = (unsigned)(r % s1);
+        const unsigned long long i0 = r / s1;
+        const T y = b[i0 * bst0 + i1 * bst1 + i2 * bst2 + (long long)i3 * bst3];
+        c[v] = from_f32<T>(to_f32<T>(a[v]) + to_f32<T>(y));
+    }
+}
+
+// ------------------------------------------------------------------ GELU
+// gelu(v) = v * (0.5 + 0.5*tanh(u)),  u = v*(0.79788456 + 0.03567741 v^2)
+//         = v * sigmoid(2u)            (no cancellation in the left tail)
+__device__ __forceinline__ float gelu_one(float v) {
+    const float u = v * (0.79788456f + 0.03567741f * v * v);
+    return v * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
+}
+
+// d/dv gelu(v) = s + 2 v s (1 - s) u',  s = sigmoid(2u),
+//   u = 0.79788456 v (1 + 0.044715 v^2),  u' = 0.79788456 + 0.1070322243 v^2
+// evaluated from e = exp(-2|u|) in (0,1] so that s and s(1-s) keep full
+// relative accuracy for large |v|.
+__device__ __forceinline__ float gelu_grad_one(float v) {
+    const float v2 = v * v;
+    const float u = 0.79788456f * v * (1.0f + 0.044715f * v2);
+    const float e = __expf(-2.0f * fabsf(u));
+    const float inv = __builtin_amdgcn_rcpf(1.0f + e);
+    const float s = u >= 0.f ? inv : e * inv;
+    const float s1ms = e * inv * inv;
+    return s + 2.0f * v * s1ms * (0.79788456f + 0.1070322243f * v2);
+}
+
+__global__ __launch_bounds__(kBlock) void gelu_fwd_f32(const float* x, float* y, int64_t n4) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) {
+        const float4 v = reinterpret_cast<const float4*>(x)[i];
+        reinterpret_cast<float4*>(y)[i] =
+            make_float4(gelu_one(v.x), gelu_one(v.y), gelu_one(v.z), gelu_one(v.w));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gelu_fwd_f16(const half8* x, half8* y, int64_t n8) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += stride) {
+        float f[8];
+        unpack8(x[i], f);
+#pragma unroll
+        for (int j = 0; j < 8; j++) f[j] = gelu_one(f[j]);
+        y[i] = pack8(f);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gelu_bwd_f32(const float* dy, const float* x, float* dx,
+                                                        int64_t n4) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n4; i += stride) {
+        const float4 v = reinterpret_cast<const float4*>(x)[i];
+        const float4 g = reinterpret_cast<const float4*>(dy)[i];
+        reinterpret_cast<float4*>(dx)[i] =
+            make_float4(g.x * gelu_grad_one(v.x), g.y * gelu_grad_one(v.y),
+                        g.z * gelu_grad_one(v.z), g.w * gelu_grad_one(v.w));
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void gelu_bwd_f16(const half8* dy, const half8* x, half8* dx,
+                                                        int64_t n8) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += stride) {
+        float v[8], g[8];
+        unpack8(x[i], v);
+        unpack8(dy[i], g);
+#pragma unroll
+        for (int j = 0; j < 8; j++) g[j] *= gelu_grad_one(v[j]);
+        dx[i] = pack8(g);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void gelu_scalar(const T* dy, const T* x, const float* bias, T* out,
+                                                       int64_t n, int64_t cols, bool backward) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        float v = to_f32<T>(x[i]);
+        if (bias) v += bias[i % cols];
+        out[i] = from_f32<T>(backward ? to_f32<T>(dy[i]) * gelu_grad_one(v) : gelu_one(v));
+    }
+}
+
+// Bias-GELU backward over a strip of rows.  A workgroup owns kBlock*VEC
+// columns and `rows_per_block` rows; each thread keeps VEC running column
+// sums of dx in registers and writes them to partial[blockIdx.y][col].
+template <typename T, int VEC>
+struct VecIO;
+template <>
+struct VecIO<float, 4> {
+    static __device__ __forceinline__ void load(const float* p, float (&f)[4]) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&f)[4]) {
+        *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+    }
+    // store, and leave in f exactly the values that were stored
+    static __device__ __forceinline__ void store_rounded(float* p, float (&f)[4]) { store(p, f); }
+};
+template <>
+struct VecIO<__half, 8> {
+    static __device__ __forceinline__ void load(const __half* p, float (&f)[8]) {
+        unpack8(*reinterpret_cast<const half8*>(p), f);
+    }
+    static __device__ __forceinline__ void store(__half* p, const float (&f)[8]) {
+        *reinterpret_cast<half8*>(p) = pack8(f);
+    }
+    // The compiler is free to fuse the producing multiply into the fp16
+    // conversion (v_fma_mixlo_f16: one rounding) for one use and not for
+    // another (v_mul_f32 + v_cvt: two roundings), which differ on rare inputs.
+    // The empty asm makes the packed registers opaque, so the store and the
+    // read-back see the very same bits.
+    static __device__ __forceinline__ void store_rounded(__half* p, float (&f)[8]) {
+        uint4 u = __builtin_bit_cast(uint4, pack8(f));
+        asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w));
+        const half8 h = __builtin_bit_cast(half8, u);
+        *reinterpret_cast<half8*>(p) = h;
+        unpack8(h, f);
+    }
+};
+
+// Bias-GELU forward with the same tiling: the VEC bias values of a thread's
+// columns stay in registers while it walks down its strip of rows.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void bias_gelu_fwd_kernel(const T* x, const float* bias, T* y,
+                                                                int64_t rows, int64_t cols,
+                                                                int rows_per_block) {
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (col >= cols) return;
+    float b[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) b[j] = bias[col + j];
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    for (int64_t r = r0; r < r1; r++) {
+        float v[VEC];
+        VecIO<T, VEC>::load(x + r * cols + col, v);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) v[j] = gelu_one(v[j] + b[j]);
+        VecIO<T, VEC>::store(y + r * cols + col, v);
+    }
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void bias_gelu_bwd_kernel(const T* dy, const T* x, const float* bias,
+                                                                T* dx, float* partial, int64_t rows,
+                                                                int64_t cols, int rows_per_block) {
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (col >= cols) return;
+    float b[VEC], acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        b[j] = bias ? bias[col + j] : 0.f;
+        acc[j] = 0.f;
+    }
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    for (int64_t r = r0; r < r1; r++) {
+        float v[VEC], g[VEC];
+        VecIO<T, VEC>::load(x + r * cols + col, v);
+        VecIO<T, VEC>::load(dy + r * cols + col, g);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            g[j] *= gelu_grad_one(v[j] + b[j]);
+        }
+        // sum what was stored, i.e. after rounding to the storage type
+        VecIO<T, VEC>::store_rounded(dx + r * cols + col, g);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) acc[j] += g[j];
+    }
+    if (partial) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) partial[(int64_t)blockIdx.y * cols + col + j] = acc[j];
+    }
+}
+
+// --------------------------------------------------------------- colsum
+// Stage 1: partial[g][c] = sum over the g-th strip of rows of x[r,c].
+template <typename T>
+__global__ __launch_bounds__(kBlock) void colsum_partial(const T* x, float* partial, int64_t rows,
+                                                          int64_t cols, int rows_per_block) {
+    const int64_t col = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (col >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    float acc = 0.f;
+    for (int64_t r = r0; r < r1; r++) acc += to_f32<T>(x[r * cols + col]);
+    partial[(int64_t)blockIdx.y * cols + col] = acc;
+}
+
+// Stage 2: out[c] = sum_g partial[g][c]  (fixed order: deterministic).
+__global__ __launch_bounds__(kBlock) void colsum_final(const float* partial, float* out, int groups,
+                                                        int64_t cols) {
+    const int64_t col = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (col >= cols) return;
+    float acc = 0.f;
+    for (int g = 0; g < groups; g++) acc += partial[(int64_t)g * cols + col];
+    out[col] = acc;
+}
+
+// ------------------------------------------------------- transpose 0213
+// One 16-byte granule per thread, indexed by OUTPUT position so stores are
+// fully coalesced; loads are contiguous runs of s3 elements.
+__global__ __launch_bounds__(kBlock) void transpose_0213_x16(const uint4* x, uint4* y, long long n16,
+                                                              unsigned s1, unsigned s2, unsigned s3g) {
+    const long long stride = (long long)gridDim.x * kBlock;
+    for (long long o = (long long)blockIdx.x * kBlock + threadIdx.x; o < n16; o += stride) {
+        unsigned long long r = (unsigned long long)o;
+        const unsigned i3 = (unsigned)(r % s3g);
+        r /= s3g;
+        const unsigned i1 = (unsigned)(r % s1);  // output dim 2 is input dim 1
+        r /= s1;
+        const unsigned i2 = (unsigned)(r % s2);
+        const unsigned long long i0 = r / s2;
+        y[o] = x[((i0 * s1 + i1) * s2 + i2) * s3g + i3];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_0213_scalar(const T* x, T* y, long long n, unsigned s1,
+                                                                 unsigned s2, unsigned s3) {
+    const long long stride = (long long)gridDim.x * kBlock;
+    for (long long o = (long long)blockIdx.x * kBlock + threadIdx.x; o < n; o += stride) {
+        unsigned long long r = (unsigned long long)o;
+        const unsigned i3 = (unsigned)(r % s3);
+        r /= s3;
+        const unsigned i1 = (unsigned)(r % s1);
+        r /= s1;
+        const unsigned i2 = (unsigned)(r % s2);
+        const unsigned long long i0 = r / s2;
+        y[o] = x[((i0 * s1 + i1) * s2 + i2) * s3 + i3];
+    }
+}
+
+// ------------------------------------------------------ data preparation
+// One workgroup per output row; rows whose id is out of range are zeroed.
+__global__ __launch_bounds__(kBlock) void gather_rows_x16(const uint4* table, const int32_t* ids, uint4* out,
+                                                           int64_t row16, int64_t vocab) {
+    const int64_t row = blockIdx.x;
+    const int64_t id = ids[row];
+    const bool ok = id >= 0 && id < vocab;
+    for (int64_t i = threadIdx.x; i < row16; i += kBlock)
+        out[row * row16 + i] = ok ? table[id * row16 + i] : make_uint4(0, 0, 0, 0);
+}
+
+__global__ __launch_bounds__(kBlock) void gather_rows_bytes(const unsigned char* table, const int32_t* ids,
+                                                             unsigned char* out, int64_t row_bytes,
+                                                             int64_t vocab) {
+    const int64_t row = blockIdx.x;
+    const int64_t id = ids[row];
+    const bool ok = id >= 0 && id < vocab;
+    for (int64_t i = threadIdx.x; i < row_bytes; i += kBlock)
+        out[row * row_bytes + i] = ok ? table[id * row_bytes + i] : (unsigned char)0;
+}
+
+constexpr int kSlopeChunk = 128;
+struct SlopeChunk {
+    double v[kSlopeChunk];
+};
+
+__global__ __launch_bounds__(kBlock) void alibi_table_kernel(float* alibi, SlopeChunk slopes, int head0,
+                                                              int nheads, int64_t tokens) {
+    const int64_t n = (int64_t)nheads * tokens;
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        const int h = (int)(i / tokens);
+        const int64_t k = i % tokens;
+        // fp64 product rounded once to fp32, as the host code it replaces does
+        alibi[(int64_t)head0 * tokens + i] = (float)((double)k * 1.0 * slopes.v[h]);
+    }
+}
+
+// One workgroup per (batch, query row).  valid = index of the first zero in
+// mask[b,:] (tokens when there is none) is found by a min-reduction.
+__global__ __launch_bounds__(kBlock) void xmask_table_kernel(const int32_t* mask, float* xmask,
+                                                              int64_t tokens) {
+    __shared__ int s_valid[kBlock / kWave];
+    const int64_t b = blockIdx.y;
+    const int64_t q = blockIdx.x;
+    const int32_t* m = mask + b * tokens;
+    int first_zero = (int)tokens;
+    // keys beyond q are masked by causality anyway, so scanning [0, q] suffices
+    for (int64_t k = threadIdx.x; k <= q; k += kBlock)
+        if (m[k] == 0 && (int)k < first_zero) first_zero = (int)k;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const int o = __shfl_xor(first_zero, off, kWave);
+        first_zero = o < first_zero ? o : first_zero;
+    }
+    if ((threadIdx.x & 63) == 0) s_valid[threadIdx.x >> 6] = first_zero;
+    __syncthreads();
+    int valid = s_valid[0];
+#pragma unroll
+    for (int w = 1; w < kBlock / kWave; w++) valid = s_valid[w] < valid ? s_valid[w] : valid;
+    float* row = xmask + (b * tokens + q) * tokens;
+    for (int64_t k = threadIdx.x; k < tokens; k += kBlock)
+        row[k] = (k <= q && k < valid) ? 0.0f : -FLT_MAX;
+}
+
+bool fits_u32(int64_t v) { return v > 0 && v <= 0xffffffffLL; }
+
+}  // namespace
+
+extern "C" {
+
+int br_hip_fill(void* dst, int dtype, float value, int64_t n, br_stream_t stream) {
+    if (n < 0) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!dst) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    const int grid = grid_for(n, kBlock);
+    switch (dtype) {
+        case BR_F32: fill_kernel<float><<<grid, kBlock, 0, st>>>((float*)dst, value, n); break;
+        case BR_F16: fill_kernel<__half><<<grid, kBlock, 0, st>>>((__half*)dst, __float2half_rn(value), n); break;
+        case BR_BF16:
+            fill_kernel<__hip_bfloat16><<<grid, kBlock, 0, st>>>((__hip_bfloat16*)dst, __float2bfloat16(value), n);
+            break;
+        case BR_I32: fill_kernel<int32_t><<<grid, kBlock, 0, st>>>((int32_t*)dst, (int32_t)value, n); break;
+        default: return BR_ERR_TODO;
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n, br_stream_t stream) {
+    if (n < 0) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!src) return BR_ERR_INPUT;
+    if (!dst) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    switch (src_dtype) {
+        case BR_F32: return cast_from<float>(src, dst, dst_dtype, n, st);
+        case BR_F16: return cast_from<__half>(src, dst, dst_dtype, n, st);
+        case BR_BF16: return cast_from<__hip_bfloat16>(src, dst, dst_dtype, n, st);
+        default: return BR_ERR_TODO;
+    }
+}
+
+int br_hip_add_bcast(const void* a, const void* b, void* c, int dtype, const int64_t as[4],
+                     const int64_t bs[4], br_stream_t stream) {
+    if (!a || !b || !as || !bs) return BR_ERR_INPUT;
+    if (!c) return BR_ERR_OUTPUT;
+    if (dtype != BR_F32 && dtype != BR_F16) return BR_ERR_TODO;
+    bool same = true;
+    for (int i = 0; i < 4; i++) {
+        if (as[i] <= 0 || bs[i] <= 0) return BR_ERR_ATTR;
+        if (bs[i] != as[i] && bs[i] != 1) return BR_ERR_INPUT;
+        same = same && bs[i] == as[i];
+    }
+    const int64_t n = as[0] * as[1] * as[2] * as[3];
+    hipStream_t st = as_stream(stream);
+    const bool al = aligned16(a) && aligned16(b) && aligned16(c);
+    if (same && al && dtype == BR_F32 && n % 4 == 0) {
+        add_same_f32x4<<<grid_for(n / 4, kBlock), kBlock, 0, st>>>((const float4*)a, (const float4*)b,
+                                                                   (float4*)c, n / 4);
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
+    }
+    if (same && al && dtype == BR_F16 && n % 8 == 0) {
+        add_same_f16x8<<<grid_for(n / 8, kBlock), kBlock, 0, st>>>((const half8*)a, (const half8*)b,
+                                                                   (half8*)c, n / 8);
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
+    }
+    if (!fits_u32(as[1]) || !fits_u32(as[2]) || !fits_u32(as[3])) return BR_ERR_ATTR;
+    const long long bst3 = bs[3] == 1 ? 0 : 1;
+    const long long bst2 = bs[2] == 1 ? 0 : bs[3];
+    const long long bst1 = bs[1] == 1 ? 0 : bs[2] * bs[3];
+    const long long bst0 = bs[0] == 1 ? 0 : bs[1] * bs[2] * bs[3];
+    // 128-bit path: needs every row start of a, b and c to stay 16-byte aligned
+    const bool vec_ok = dtype == BR_F32 && al && as[3] % 4 == 0 && (bst3 == 0 || bs[3] % 4 == 0);
+    if (vec_ok) {
+        BcastDims d;
+        d.s1 = (unsigned)as[1];
+        d.s2 = (unsigned)as[2];
+        d.s3v = (unsigned)(as[3] / 4);
+        d.bst0 = bst0; d.bst1 = bst1; d.bst2 = bst2; d.bst3 = (int)bst3;
+        add_bcast_f32x4<<<grid_for(n / 4, kBlock), kBlock, 0, st>>>((const float*)a, (const float*)b,
+                                                                    (float*)c, n / 4, d);
+    } else if (dtype == BR_F32) {
+        add_bcast_scalar<float><<<grid_for(n, kBlock), kBlock, 0, st>>>(
+            (const float*)a, (const float*)b, (float*)c, n, (unsigned)as[1], (unsigned)as[2],
+            (unsigned)as[3], bst0, bst1, bst2, (int)bst3);
+    } else {
+        add_bcast_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>(
+            (const __half*)a, (const __half*)b, (__half*)c, n, (unsigned)as[1], (unsigned)as[2],
+            (unsigned)as[3], bst0, bst1, bst2, (int)bst3);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+static int strip_rows(int64_t rows) {
+    // strips of rows per workgroup: about 64 strips, at least 8 rows each
+    int64_t rpb = (rows + 63) / 64;
+    if (rpb < 8) rpb = 8;
+    return (int)rpb;
+}
+
+int br_hip_gelu_fwd(const void* x, void* y, int dtype, int64_t n, br_stream_t stream) {
+    if (n < 0) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!x) return BR_ERR_INPUT;
+    if (!y) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    const bool al = aligned16(x) && aligned16(y);
+    if (dtype == BR_F32 && al && n % 4 == 0) {
+        gelu_fwd_f32<<<grid_for(n / 4, kBlock), kBlock, 0, st>>>((const float*)x, (float*)y, n / 4);
+    } else if (dtype == BR_F16 && al && n % 8 == 0) {
+        gelu_fwd_f16<<<grid_for(n / 8, kBlock), kBlock, 0, st>>>((const half8*)x, (half8*)y, n / 8);
+    } else if (dtype == BR_F32) {
+        gelu_scalar<float><<<grid_for(n, kBlock), kBlock, 0, st>>>(nullptr, (const float*)x, nullptr, (float*)y,
+                                                                  n, 1, false);
+    } else if (dtype == BR_F16) {
+        gelu_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>(nullptr, (const __half*)x, nullptr,
+                                                                   (__half*)y, n, 1, false);
+    } else {
+        return BR_ERR_TODO;
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_bias_gelu_fwd(const void* x, const float* bias, void* y, int dtype, int64_t rows, int64_t cols,
+                         br_stream_t stream) {
+    if (rows < 0 || cols <= 0) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!x || !bias) return BR_ERR_INPUT;
+    if (!y) return BR_ERR_OUTPUT;
+    if (dtype != BR_F32 && dtype != BR_F16) return BR_ERR_TODO;
+    hipStream_t st = as_stream(stream);
+    const int rpb = strip_rows(rows);
+    const unsigned groups = (unsigned)((rows + rpb - 1) / rpb);
+    const bool al = aligned16(x) && aligned16(y);
+    if (dtype == BR_F32 && al && cols % 4 == 0) {
+        dim3 grid((unsigned)((cols / 4 + kBlock - 1) / kBlock), groups);
+        bias_gelu_fwd_kernel<float, 4><<<grid, kBlock, 0, st>>>((const float*)x, bias, (float*)y, rows, cols, rpb);
+    } else if (dtype == BR_F16 && al && cols % 8 == 0) {
+        dim3 grid((unsigned)((cols / 8 + kBlock - 1) / kBlock), groups);
+        bias_gelu_fwd_kernel<__half, 8><<<grid, kBlock, 0, st>>>((const __half*)x, bias, (__half*)y, rows, cols,
+                                                                  rpb);
+    } else {
+        const int64_t n = rows * cols;
+        if (dtype == BR_F32)
+            gelu_scalar<float><<<grid_for(n, kBlock), kBlock, 0, st>>>(nullptr, (const float*)x, bias, (float*)y,
+                                                                      n, cols, false);
+        else
+            gelu_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>(nullptr, (const __half*)x, bias,
+                                                                       (__half*)y, n, cols, false);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_gelu_bwd(const void* dy, const void* x, void* dx, int dtype, int64_t n, br_stream_t stream) {
+    if (n < 0) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!dy || !x) return BR_ERR_INPUT;
+    if (!dx) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    const bool al = aligned16(dy) && aligned16(x) && aligned16(dx);
+    if (dtype == BR_F32 && al && n % 4 == 0) {
+        gelu_bwd_f32<<<grid_for(n / 4, kBlock), kBlock, 0, st>>>((const float*)dy, (const float*)x, (float*)dx,
+                                                                n / 4);
+    } else if (dtype == BR_F16 && al && n % 8 == 0) {
+        gelu_bwd_f16<<<grid_for(n / 8, kBlock), kBlock, 0, st>>>((const half8*)dy, (const half8*)x, (half8*)dx,
+                                                                n / 8);
+    } else if (dtype == BR_F32) {
+        gelu_scalar<float><<<grid_for(n, kBlock), kBlock, 0, st>>>((const float*)dy, (const float*)x, nullptr,
+                                                                  (float*)dx, n, 1, true);
+    } else if (dtype == BR_F16) {
+        gelu_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>((const __half*)dy, (const __half*)x, nullptr,
+                                                                   (__half*)dx, n, 1, true);
+    } else {
+        return BR_ERR_TODO;
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+size_t br_hip_bias_gelu_bwd_workspace(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    const int rpb = strip_rows(rows);
+    const int64_t groups = (rows + rpb - 1) / rpb;
+    return (size_t)(groups * cols) * sizeof(float);
+}
+
+int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void* dx, float* dbias, int dtype,
+                         int64_t rows, int64_t cols, void* workspace, size_t workspace_bytes,
+                         br_stream_t stream) {
+    if (rows < 0 || cols <= 0) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!dy || !x) return BR_ERR_INPUT;
+    if (!dx) return BR_ERR_OUTPUT;
+    if (dtype != BR_F32 && dtype != BR_F16) return BR_ERR_TODO;
+    hipStream_t st = as_stream(stream);
+    const int rpb = strip_rows(rows);
+    const int groups = (int)((rows + rpb - 1) / rpb);
+    float* partial = nullptr;
+    if (dbias) {
+        if (!workspace || workspace_bytes < br_hip_bias_gelu_bwd_workspace(rows, cols)) return BR_ERR_ATTR;
+        partial = (float*)workspace;
+    }
+    const bool al = aligned16(dy) && aligned16(x) && aligned16(dx);
+    if (dtype == BR_F32 && al && cols % 4 == 0) {
+        dim3 grid((unsigned)((cols / 4 + kBlock - 1) / kBlock), (unsigned)groups);
+        bias_gelu_bwd_kernel<float, 4><<<grid, kBlock, 0, st>>>((const float*)dy, (const float*)x, bias,
+                                                                 (float*)dx, partial, rows, cols, rpb);
+    } else if (dtype == BR_F16 && al && cols % 8 == 0) {
+        dim3 grid((unsigned)((cols / 8 + kBlock - 1) / kBlock), (unsigned)groups);
+        bias_gelu_bwd_kernel<__half, 8><<<grid, kBlock, 0, st>>>((const __half*)dy, (const __half*)x, bias,
+                                                                  (__half*)dx, partial, rows, cols, rpb);
+    } else {
+        // unaligned shapes: elementwise pass, then a separate column sum of dx
+        const int64_t n = rows * cols;
+        if (dtype == BR_F32)
+            gelu_scalar<float><<<grid_for(n, kBlock), kBlock, 0, st>>>((const float*)dy, (const float*)x, bias,
+                                                                      (float*)dx, n, cols, true);
+        else
+            gelu_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>((const __half*)dy, (const __half*)x,
+                                                                       bias, (__half*)dx, n, cols, true);
+        BR_HIP_LAUNCH_CHECK();
+        if (dbias) return br_hip_colsum(dx, dtype, dbias, rows, cols, workspace, workspace_bytes, stream);
+        return BR_OK;
+    }
+    BR_HIP_LAUNCH_CHECK();
+    if (dbias) {
+        colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>(partial, dbias, groups, cols);
+        BR_HIP_LAUNCH_CHECK();
+    }
+    return BR_OK;
+}
+
+size_t br_hip_colsum_workspace(int64_t rows, int64_t cols) {
+    return br_hip_bias_gelu_bwd_workspace(rows, cols);
+}
+
+int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols, void* workspace,
+                  size_t workspace_bytes, br_stream_t stream) {
+    if (rows < 0 || cols <= 0) return BR_ERR_ATTR;
+    if (!out) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    if (rows == 0) return br_hip_fill(out, BR_F32, 0.f, cols, stream);
+    if (!x) return BR_ERR_INPUT;
+    if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
+    const int rpb = strip_rows(rows);
+    const int groups = (int)((rows + rpb - 1) / rpb);
+    dim3 grid((unsigned)((cols + kBlock - 1) / kBlock), (unsigned)groups);
+    if (dtype == BR_F32)
+        colsum_partial<float><<<grid, kBlock, 0, st>>>((const float*)x, (float*)workspace, rows, cols, rpb);
+    else if (dtype == BR_F16)
+        colsum_partial<__half><<<grid, kBlock, 0, st>>>((const __half*)x, (float*)workspace, rows, cols, rpb);
+    else
+        return BR_ERR_TODO;
+    BR_HIP_LAUNCH_CHECK();
+    colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>((const float*)workspace, out,
+                                                                               groups, cols);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, int64_t s1, int64_t s2,
+                          int64_t s3, br_stream_t stream) {
+    if (s0 < 0 || s1 <= 0 || s2 <= 0 || s3 <= 0) return BR_ERR_ATTR;
+    if (elem_bytes != 2 && elem_bytes != 4) return BR_ERR_ATTR;
+    if (s0 == 0) return BR_OK;
+    if (!x) return BR_ERR_INPUT;
+    if (!y || x == y) return BR_ERR_OUTPUT;
+    if (!fits_u32(s1) || !fits_u32(s2) || !fits_u32(s3)) return BR_ERR_ATTR;
+    hipStream_t st = as_stream(stream);
+    const int64_t n = s0 * s1 * s2 * s3;
+    const int per16 = 16 / elem_bytes;
+    if (s3 % per16 == 0 && aligned16(x) && aligned16(y)) {
+        const int64_t n16 = n / per16;
+        transpose_0213_x16<<<grid_for(n16, kBlock), kBlock, 0, st>>>((const uint4*)x, (uint4*)y, n16,
+                                                                    (unsigned)s1, (unsigned)s2,
+                                                                    (unsigned)(s3 / per16));
+    } else if (elem_bytes == 4) {
+        transpose_0213_scalar<uint32_t><<<grid_for(n, kBlock), kBlock, 0, st>>>(
+            (const uint32_t*)x, (uint32_t*)y, n, (unsigned)s1, (unsigned)s2, (unsigned)s3);
+    } else {
+        transpose_0213_scalar<uint16_t><<<grid_for(n, kBlock), kBlock, 0, st>>>(
+            (const uint16_t*)x, (uint16_t*)y, n, (unsigned)s1, (unsigned)s2, (unsigned)s3);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, int elem_bytes, int64_t n,
+                            int64_t hidden, int64_t vocab, br_stream_t stream) {
+    if (n < 0 || hidden <= 0 || vocab <= 0 || (elem_bytes != 2 && elem_bytes != 4)) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!table || !ids) return BR_ERR_INPUT;
+    if (!out) return BR_ERR_OUTPUT;
+    if (n > 0x7fffffff) return BR_ERR_ATTR;
+    hipStream_t st = as_stream(stream);
+    const int64_t row_bytes = hidden * elem_bytes;
+    if (row_bytes % 16 == 0 && aligned16(table) && aligned16(out))
+        gather_rows_x16<<<(unsigned)n, kBlock, 0, st>>>((const uint4*)table, ids, (uint4*)out, row_bytes / 16,
+                                                        vocab);
+    else
+        gather_rows_bytes<<<(unsigned)n, kBlock, 0, st>>>((const unsigned char*)table, ids, (unsigned char*)out,
+                                                          row_bytes, vocab);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_alibi_table(float* alibi, int64_t heads, int64_t tokens, br_stream_t stream) {
+    if (heads <= 0 || tokens <= 0 || heads > 65536) return BR_ERR_ATTR;
+    if (!alibi) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    double* slopes = new double[heads];
+    br_hip_alibi_slopes(slopes, heads);
+    int rc = BR_OK;
+    for (int64_t h0 = 0; h0 < heads && rc == BR_OK; h0 += kSlopeChunk) {
+        SlopeChunk c;
+        const int nh = (int)(heads - h0 < kSlopeChunk ? heads - h0 : kSlopeChunk);
+        for (int i = 0; i < kSlopeChunk; i++) c.v[i] = i < nh ? slopes[h0 + i] : 0.0;
+        alibi_table_kernel<<<grid_for((int64_t)nh * tokens, kBlock), kBlock, 0, st>>>(alibi, c, (int)h0, nh,
+                                                                                      tokens);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) rc = (int)e;
+    }
+    delete[] slopes;
+    return rc;
+}
+
+int br_hip_xmask_table(const int32_t* mask, float* xmask, int64_t batch, int64_t tokens, br_stream_t stream) {
+    if (batch < 0 || tokens <= 0 || tokens > 0x7fffffff || batch > 65535) return BR_ERR_ATTR;
+    if (batch == 0) return BR_OK;
+    if (!mask) return BR_ERR_INPUT;
+    if (!xmask) return BR_ERR_OUTPUT;
+    dim3 grid((unsigned)tokens, (unsigned)batch);
+    xmask_table_kernel<<<grid, kBlock, 0, as_stream(stream)>>>(mask, xmask, tokens);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+}  // extern "C"

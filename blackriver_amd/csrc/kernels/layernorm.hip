@@ -1,0 +1,358 @@
+// LayerNorm forward / backward for gfx950.
+//
+// Forward: one 256-thread workgroup per row; the row is read from HBM once
+// into registers (128-bit loads), mean and centred variance are reduced with
+// wave64 butterflies plus one LDS exchange, and the normalised row is written
+// straight from registers.
+//
+// Backward: persistent workgroups walk over rows.  Each thread keeps gamma,
+// beta and running dgamma / dbeta sums for its own columns in registers, so
+// dy and y are read exactly once; per-workgroup partial column sums go to a
+// workspace and a small second kernel adds them in a fixed order.
+#include "common.hpp"
+
+using namespace brk;
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+
+__device__ __forceinline__ float add_eps(float g, float eps) {
+    return fabsf(g) > eps ? g : (g < 0.f ? -eps : eps);
+}
+
+// ---------------------------------------------------------------- forward
+// VPT = float4 vectors per thread; cols4 = cols / 4 <= kBlock * VPT.
+template <int VPT>
+__global__ __launch_bounds__(kBlock) void ln_fwd_regs(const float* __restrict__ x,
+                                                       const float* __restrict__ gamma,
+                                                       const float* __restrict__ beta,
+                                                       float* __restrict__ y, float* __restrict__ mean_out,
+                                                       float* __restrict__ var_out, int cols4, float eps,
+                                                       float inv_cols) {
+    __shared__ float lds[2][kWaves];
+    const int64_t row = blockIdx.x;
+    const float4* xr = reinterpret_cast<const float4*>(x) + row * cols4;
+    float4 v[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * kBlock;
+        v[i] = idx < cols4 ? xr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float s[1] = {0.f};
+#pragma unroll
+    for (int i = 0; i < VPT; i++) s[0] += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    block_sum<1>(s, lds[0]);
+    const float mean = s[0] * inv_cols;
+
+    float q[1] = {0.f};
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * kBlock;
+        if (idx < cols4) {
+            const float a = v[i].x - mean, b = v[i].y - mean, c = v[i].z - mean, d = v[i].w - mean;
+            q[0] += (a * a + b * b) + (c * c + d * d);
+        }
+    }
+    block_sum<1>(q, lds[1]);
+    const float var = q[0] * inv_cols + eps;  // the stored statistic includes eps
+    const float rstd = 1.0f / sqrtf(var);
+    if (threadIdx.x == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (var_out) var_out[row] = var;
+    }
+    float4* yr = reinterpret_cast<float4*>(y) + row * cols4;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * kBlock;
+        if (idx < cols4) {
+            const float4 g = reinterpret_cast<const float4*>(gamma)[idx];
+            const float4 b = reinterpret_cast<const float4*>(beta)[idx];
+            float4 o;
+            o.x = (v[i].x - mean) * rstd * g.x + b.x;
+            o.y = (v[i].y - mean) * rstd * g.y + b.y;
+            o.z = (v[i].z - mean) * rstd * g.z + b.z;
+            o.w = (v[i].w - mean) * rstd * g.w + b.w;
+            yr[idx] = o;
+        }
+    }
+}
+
+// Any width / alignment: three sweeps over the row from global memory.
+__global__ __launch_bounds__(kBlock) void ln_fwd_generic(const float* x, const float* gamma, const float* beta,
+                                                          float* y, float* mean_out, float* var_out,
+                                                          int64_t cols, float eps) {
+    __shared__ float lds[2][kWaves];
+    const int64_t row = blockIdx.x;
+    const float* xr = x + row * cols;
+    float s[1] = {0.f};
+    for (int64_t c = threadIdx.x; c < cols; c += kBlock) s[0] += xr[c];
+    block_sum<1>(s, lds[0]);
+    const float mean = s[0] / (float)cols;
+    float q[1] = {0.f};
+    for (int64_t c = threadIdx.x; c < cols; c += kBlock) {
+        const float d = xr[c] - mean;
+        q[0] += d * d;
+    }
+    block_sum<1>(q, lds[1]);
+    const float var = q[0] / (float)cols + eps;
+    const float rstd = 1.0f / sqrtf(var);
+    if (threadIdx.x == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (var_out) var_out[row] = var;
+    }
+    for (int64_t c = threadIdx.x; c < cols; c += kBlock)
+        y[row * cols + c] = (xr[c] - mean) * rstd * gamma[c] + beta[c];
+}
+
+// --------------------------------------------------------------- backward
+template <int VPT>
+__global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* __restrict__ dy, const float* __restrict__ y,
+                                                       const float* __restrict__ gamma,
+                                                       const float* __restrict__ beta,
+                                                       const float* __restrict__ var, float* __restrict__ dx,
+                                                       float* __restrict__ part_dgamma,
+                                                       float* __restrict__ part_dbeta, int64_t rows, int cols4,
+                                                       float eps, float inv_cols) {
+    __shared__ float lds[2][2 * kWaves];
+    float4 g[VPT], ginv[VPT], b[VPT], acc_g[VPT], acc_b[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * kBlock;
+        const bool ok = idx < cols4;
+        g[i] = ok ? reinterpret_cast<const float4*>(gamma)[idx] : make_float4(1.f, 1.f, 1.f, 1.f);
+        b[i] = ok ? reinterpret_cast<const float4*>(beta)[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+        ginv[i] = make_float4(1.0f / add_eps(g[i].x, eps), 1.0f / add_eps(g[i].y, eps),
+                              1.0f / add_eps(g[i].z, eps), 1.0f / add_eps(g[i].w, eps));
+        acc_g[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        acc_b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    int flip = 0;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, flip ^= 1) {
+        const float4* dyr = reinterpret_cast<const float4*>(dy) + row * cols4;
+        const float4* yr = reinterpret_cast<const float4*>(y) + row * cols4;
+        float4 d[VPT], xh[VPT];
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int idx = threadIdx.x + i * kBlock;
+            const bool ok = idx < cols4;
+            d[i] = ok ? dyr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+            xh[i] = ok ? yr[idx] : b[i];
+        }
+        // stored var already holds eps; the backward adds eps once more
+        const float rstd = 1.0f / sqrtf(var[row] + eps);
+        float s[2] = {0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            xh[i].x = (xh[i].x - b[i].x) * ginv[i].x;
+            xh[i].y = (xh[i].y - b[i].y) * ginv[i].y;
+            xh[i].z = (xh[i].z - b[i].z) * ginv[i].z;
+            xh[i].w = (xh[i].w - b[i].w) * ginv[i].w;
+            acc_b[i].x += d[i].x; acc_b[i].y += d[i].y; acc_b[i].z += d[i].z; acc_b[i].w += d[i].w;
+            acc_g[i].x += d[i].x * xh[i].x; acc_g[i].y += d[i].y * xh[i].y;
+            acc_g[i].z += d[i].z * xh[i].z; acc_g[i].w += d[i].w * xh[i].w;
+            // from here on d holds dxhat = dy * gamma
+            d[i].x *= g[i].x; d[i].y *= g[i].y; d[i].z *= g[i].z; d[i].w *= g[i].w;
+            s[0] += (d[i].x + d[i].y) + (d[i].z + d[i].w);
+            s[1] += (d[i].x * xh[i].x + d[i].y * xh[i].y) + (d[i].z * xh[i].z + d[i].w * xh[i].w);
+        }
+        block_sum<2>(s, lds[flip]);
+        const float m1 = s[0] * inv_cols, m2 = s[1] * inv_cols;
+        float4* dxr = reinterpret_cast<float4*>(dx) + row * cols4;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int idx = threadIdx.x + i * kBlock;
+            if (idx < cols4) {
+                float4 o;
+                o.x = (d[i].x - m1 - xh[i].x * m2) * rstd;
+                o.y = (d[i].y - m1 - xh[i].y * m2) * rstd;
+                o.z = (d[i].z - m1 - xh[i].z * m2) * rstd;
+                o.w = (d[i].w - m1 - xh[i].w * m2) * rstd;
+                dxr[idx] = o;
+            }
+        }
+    }
+    float4* pg = reinterpret_cast<float4*>(part_dgamma) + (int64_t)blockIdx.x * cols4;
+    float4* pb = reinterpret_cast<float4*>(part_dbeta) + (int64_t)blockIdx.x * cols4;
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int idx = threadIdx.x + i * kBlock;
+        if (idx < cols4) {
+            pg[idx] = acc_g[i];
+            pb[idx] = acc_b[i];
+        }
+    }
+}
+
+// Any width / alignment: row pass from global memory (dx only).
+__global__ __launch_bounds__(kBlock) void ln_bwd_dx_generic(const float* dy, const float* y, const float* gamma,
+                                                             const float* beta, const float* var, float* dx,
+                                                             int64_t cols, float eps) {
+    __shared__ float lds[2 * kWaves];
+    const int64_t row = blockIdx.x;
+    const float rstd = 1.0f / sqrtf(var[row] + eps);
+    float s[2] = {0.f, 0.f};
+    for (int64_t c = threadIdx.x; c < cols; c += kBlock) {
+        const float dxhat = dy[row * cols + c] * gamma[c];
+        const float xhat = (y[row * cols + c] - beta[c]) / add_eps(gamma[c], eps);
+        s[0] += dxhat;
+        s[1] += dxhat * xhat;
+    }
+    block_sum<2>(s, lds);
+    const float m1 = s[0] / (float)cols, m2 = s[1] / (float)cols;
+    for (int64_t c = threadIdx.x; c < cols; c += kBlock) {
+        const float dxhat = dy[row * cols + c] * gamma[c];
+        const float xhat = (y[row * cols + c] - beta[c]) / add_eps(gamma[c], eps);
+        dx[row * cols + c] = (dxhat - m1 - xhat * m2) * rstd;
+    }
+}
+
+// Any width: partial column sums over a strip of rows, one column per thread.
+__global__ __launch_bounds__(kBlock) void ln_bwd_cols_generic(const float* dy, const float* y, const float* gamma,
+                                                               const float* beta, float* part_dgamma,
+                                                               float* part_dbeta, int64_t rows, int64_t cols,
+                                                               int rows_per_block, float eps) {
+    const int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (c >= cols) return;
+    const float ginv = 1.0f / add_eps(gamma[c], eps), b = beta[c];
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    float sg = 0.f, sb = 0.f;
+    for (int64_t r = r0; r < r1; r++) {
+        const float d = dy[r * cols + c];
+        sb += d;
+        sg += d * ((y[r * cols + c] - b) * ginv);
+    }
+    part_dgamma[(int64_t)blockIdx.y * cols + c] = sg;
+    part_dbeta[(int64_t)blockIdx.y * cols + c] = sb;
+}
+
+// dgamma[c] = sum_p part_dgamma[p][c] (and dbeta likewise), fixed order.
+// blockDim = (64 columns, 4 slices of partials); slices are combined in LDS.
+__global__ __launch_bounds__(kBlock) void ln_bwd_finalize(const float* part_dgamma, const float* part_dbeta,
+                                                           float* dgamma, float* dbeta, int parts, int64_t cols) {
+    __shared__ float lg[4][64], lb[4][64];
+    const int cx = threadIdx.x & 63, sl = threadIdx.x >> 6;
+    const int64_t c = (int64_t)blockIdx.x * 64 + cx;
+    float sg = 0.f, sb = 0.f;
+    if (c < cols) {
+        for (int p = sl; p < parts; p += 4) {
+            sg += part_dgamma[(int64_t)p * cols + c];
+            sb += part_dbeta[(int64_t)p * cols + c];
+        }
+    }
+    lg[sl][cx] = sg;
+    lb[sl][cx] = sb;
+    __syncthreads();
+    if (sl == 0 && c < cols) {
+        dgamma[c] = (lg[0][cx] + lg[1][cx]) + (lg[2][cx] + lg[3][cx]);
+        dbeta[c] = (lb[0][cx] + lb[1][cx]) + (lb[2][cx] + lb[3][cx]);
+    }
+}
+
+int bwd_parts(int64_t rows) {
+    // persistent workgroups: two per CU on a 256-CU part, never more than rows
+    int64_t p = 512;
+    if (p > rows) p = rows;
+    return (int)(p < 1 ? 1 : p);
+}
+
+int strip_rows(int64_t rows) {
+    int64_t rpb = (rows + 127) / 128;
+    if (rpb < 8) rpb = 8;
+    return (int)rpb;
+}
+
+bool regs_path_ok(int64_t cols, const void* a, const void* b, const void* c, const void* d, const void* e) {
+    return cols % 4 == 0 && cols / 4 <= kBlock * 8 && aligned16(a) && aligned16(b) && aligned16(c) &&
+           aligned16(d) && aligned16(e);
+}
+
+}  // namespace
+
+extern "C" {
+
+int br_hip_layernorm_fwd(const float* x, const float* gamma, const float* beta, float* y, float* mean,
+                         float* var, int64_t rows, int64_t cols, float eps, br_stream_t stream) {
+    if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!x || !gamma || !beta) return BR_ERR_INPUT;
+    if (!y) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    const unsigned grid = (unsigned)rows;
+    if (regs_path_ok(cols, x, gamma, beta, y, y)) {
+        const int cols4 = (int)(cols / 4);
+        const float inv = 1.0f / (float)cols;
+        const int vpt = (cols4 + kBlock - 1) / kBlock;
+        if (vpt <= 1)
+            ln_fwd_regs<1><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
+        else if (vpt <= 2)
+            ln_fwd_regs<2><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
+        else if (vpt <= 4)
+            ln_fwd_regs<4><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
+        else
+            ln_fwd_regs<8><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
+    } else {
+        ln_fwd_generic<<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols, eps);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    int64_t parts = bwd_parts(rows);
+    const int64_t strips = (rows + strip_rows(rows) - 1) / strip_rows(rows);
+    if (strips > parts) parts = strips;
+    return (size_t)(2 * parts * cols) * sizeof(float);
+}
+
+int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, const float* beta,
+                         const float* var, float* dgamma, float* dbeta, float* dx, int64_t rows, int64_t cols,
+                         float eps, void* workspace, size_t workspace_bytes, br_stream_t stream) {
+    if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
+    if (!dgamma || !dbeta) return BR_ERR_OUTPUT;
+    if (rows == 0) {
+        int rc = br_hip_fill(dgamma, BR_F32, 0.f, cols, stream);
+        return rc ? rc : br_hip_fill(dbeta, BR_F32, 0.f, cols, stream);
+    }
+    if (!dy || !y || !gamma || !beta || !var) return BR_ERR_INPUT;
+    if (!dx) return BR_ERR_OUTPUT;
+    if (!workspace || workspace_bytes < br_hip_layernorm_bwd_workspace(rows, cols)) return BR_ERR_ATTR;
+    hipStream_t st = as_stream(stream);
+    int parts;
+    float* part_g = (float*)workspace;
+    if (regs_path_ok(cols, dy, y, gamma, beta, dx) && aligned16(workspace)) {
+        parts = bwd_parts(rows);
+        float* part_b = part_g + (int64_t)parts * cols;
+        const int cols4 = (int)(cols / 4);
+        const float inv = 1.0f / (float)cols;
+        const int vpt = (cols4 + kBlock - 1) / kBlock;
+        if (vpt <= 1)
+            ln_bwd_regs<1><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+        else if (vpt <= 2)
+            ln_bwd_regs<2><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+        else if (vpt <= 4)
+            ln_bwd_regs<4><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+        else
+            ln_bwd_regs<8><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+        BR_HIP_LAUNCH_CHECK();
+        ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols);
+    } else {
+        const int rpb = strip_rows(rows);
+        parts = (int)((rows + rpb - 1) / rpb);
+        float* part_b = part_g + (int64_t)parts * cols;
+        dim3 grid((unsigned)((cols + kBlock - 1) / kBlock), (unsigned)parts);
+        // column sums first: they read dy, which dx must not have replaced yet
+        ln_bwd_cols_generic<<<grid, kBlock, 0, st>>>(dy, y, gamma, beta, part_g, part_b, rows, cols, rpb, eps);
+        BR_HIP_LAUNCH_CHECK();
+        ln_bwd_dx_generic<<<(unsigned)rows, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, cols, eps);
+        BR_HIP_LAUNCH_CHECK();
+        ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,229 @@
+/*
+ * br_hip.h -- C ABI of libbr_hip.so, the MI355X (gfx950) kernel library
+ * behind BlackRiver's tensor operator API.
+ *
+ * One entry point per kernel family.  Every function takes raw device
+ * pointers, explicit sizes and the HIP stream to launch on (a hipStream_t
+ * passed as void*; NULL is the default stream) and returns 0 on success, a
+ * positive hipError_t value when the HIP runtime failed, or a negative
+ * BR_ERR_* value when the arguments are rejected before any launch.  Nothing
+ * here allocates device memory except br_hip_malloc / br_hip_host_malloc;
+ * kernels that need scratch take a caller-provided workspace.
+ *
+ * Tensors are dense row-major.  "dtype" arguments use the numbering of the
+ * reference's br::DataType (blackriver/tensortype.hpp:16-21).
+ *
+ * Each declaration cites the reference interface it stands in for (paths
+ * relative to the reference tree).
+ */
+#ifndef BR_HIP_H_
+#define BR_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* br_stream_t; /* hipStream_t */
+typedef void* br_event_t;  /* hipEvent_t  */
+
+enum {
+    BR_F32 = 0,
+    BR_BF16 = 1,
+    BR_F16 = 2,
+    BR_I32 = 3
+};
+
+enum {
+    BR_OK = 0,
+    BR_ERR_TODO = -1,     /* combination not implemented  (OP_TODO_ERROR)   */
+    BR_ERR_INPUT = -2,    /* bad input argument           (OP_INPUT_ERROR)  */
+    BR_ERR_OUTPUT = -3,   /* bad output argument          (OP_OUTPUT_ERROR) */
+    BR_ERR_ATTR = -4      /* bad scalar attribute / size  (OP_ATTR_ERROR)   */
+};
+
+/* ---- runtime plumbing -------------------------------------------------- */
+/* Stand in for the CUDA runtime calls of blackriver/context.cpp:18-43
+ * (cudaSetDevice, cudaStreamCreate, cudaMalloc of the workspace) and of
+ * blackriver/cuda_tensor.hpp:11-20 (cudaMalloc / cudaFree per tensor). */
+int br_hip_device_count(int* count);
+int br_hip_set_device(int device);
+const char* br_hip_error_string(int code);
+int br_hip_malloc(void** ptr, size_t bytes);
+int br_hip_free(void* ptr);
+int br_hip_host_malloc(void** ptr, size_t bytes); /* pinned host memory */
+int br_hip_host_free(void* ptr);
+int br_hip_stream_create(br_stream_t* stream);
+int br_hip_stream_destroy(br_stream_t stream);
+int br_hip_stream_sync(br_stream_t stream); /* nn.cpp:16-22 (op.sync) */
+int br_hip_event_create(br_event_t* event);
+int br_hip_event_destroy(br_event_t event);
+int br_hip_event_record(br_event_t event, br_stream_t stream);
+int br_hip_event_sync(br_event_t event);
+int br_hip_event_elapsed_ms(br_event_t start, br_event_t stop, float* ms);
+
+/* cudaMemcpyAsync in cuda_tensor.cpp:135,139 and cpu_tensor.cpp:31, and
+ * cudaMemset in cuda_tensor.cpp:104.  Asynchronous on `stream`. */
+int br_hip_memcpy_h2d(void* dst, const void* src, size_t bytes, br_stream_t stream);
+int br_hip_memcpy_d2h(void* dst, const void* src, size_t bytes, br_stream_t stream);
+int br_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, br_stream_t stream);
+int br_hip_memset(void* dst, int byte_value, size_t bytes, br_stream_t stream);
+
+/* ---- elementwise ------------------------------------------------------- */
+/* cudnnSetTensor in cuda_tensor.cpp:111-125 (op_fill). */
+int br_hip_fill(void* dst, int dtype, float value, int64_t n, br_stream_t stream);
+
+/* Storage conversion between BR_F32, BR_F16 and BR_BF16 (no counterpart in
+ * the reference, whose only implemented dtype is fp32). */
+int br_hip_cast(const void* src, int src_dtype, void* dst, int dst_dtype, int64_t n,
+                br_stream_t stream);
+
+/* cudnnOpTensor(ADD) in cuda_tensor.cpp:206-232 (op_add): c = a + b where b
+ * is broadcast along every dimension in which b_shape is 1.  Shapes are
+ * rank 4 (lower ranks mapped as cuda_tensor.hpp:39-49).  c may alias a. */
+int br_hip_add_bcast(const void* a, const void* b, void* c, int dtype,
+                     const int64_t a_shape[4], const int64_t b_shape[4], br_stream_t stream);
+
+/* kernels::gelu_forward / gelu_backward, kernels/gelu.cu:46-59,72-85
+ * (declared kernels/kernels.h:518-519), called at cuda_tensor.cpp:400-412,814-828.
+ * dtype is the storage type of x / y / dy / dx (BR_F32 or BR_F16); math is
+ * fp32.  dx may alias x. */
+int br_hip_gelu_fwd(const void* x, void* y, int dtype, int64_t n, br_stream_t stream);
+int br_hip_gelu_bwd(const void* dy, const void* x, void* dx, int dtype, int64_t n,
+                    br_stream_t stream);
+
+/* y = gelu(x + bias[col]): the cudnnAddTensor bias pass of
+ * cuda_tensor.cpp:180-190 fused with kernels::gelu_forward.  bias is fp32. */
+int br_hip_bias_gelu_fwd(const void* x, const float* bias, void* y, int dtype, int64_t rows,
+                         int64_t cols, br_stream_t stream);
+/* dx = dy * gelu'(x + bias); when dbias != NULL also dbias[col] = sum_rows dx
+ * (the cudnnReduceTensor of cuda_tensor.cpp:738-760).  workspace must hold
+ * br_hip_bias_gelu_bwd_workspace(rows, cols) bytes when dbias != NULL. */
+size_t br_hip_bias_gelu_bwd_workspace(int64_t rows, int64_t cols);
+int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void* dx,
+                         float* dbias, int dtype, int64_t rows, int64_t cols, void* workspace,
+                         size_t workspace_bytes, br_stream_t stream);
+
+/* kernels::launch_transform_0213<float>, kernels/transform_kernels.cu:56-65
+ * (declared kernels/kernels.h:35), called at cuda_tensor.cpp:257-275: [s0,s1,s2,s3] -> [s0,s2,s1,s3].
+ * elem_bytes is 2 or 4. */
+int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, int64_t s1,
+                          int64_t s2, int64_t s3, br_stream_t stream);
+
+/* cudnnReduceTensor(ADD) of cuda_tensor.cpp:738-760: out[c] = sum_r x[r,c]
+ * (x fp32 or fp16, out fp32).  workspace: br_hip_colsum_workspace bytes. */
+size_t br_hip_colsum_workspace(int64_t rows, int64_t cols);
+int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols,
+                  void* workspace, size_t workspace_bytes, br_stream_t stream);
+
+/* ---- LayerNorm --------------------------------------------------------- */
+/* kernels::launch_layer_norm_float, kernels/normalize_kernels.cu:87-102
+ * (declared kernels/kernels.h:24), called at cuda_tensor.cpp:236-255.  var receives sigma^2 + eps; mean and
+ * var may be NULL. */
+int br_hip_layernorm_fwd(const float* x, const float* gamma, const float* beta, float* y,
+                         float* mean, float* var, int64_t rows, int64_t cols, float eps,
+                         br_stream_t stream);
+
+/* kernels::launch_ln_bw_float, kernels/normalize_kernels.cu:361-383
+ * (declared kernels/kernels.h:28) with means == nullptr, called at cuda_tensor.cpp:699-727.  y is the forward
+ * OUTPUT, var what the forward stored; dgamma / dbeta are overwritten. */
+size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols);
+int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma,
+                         const float* beta, const float* var, float* dgamma, float* dbeta,
+                         float* dx, int64_t rows, int64_t cols, float eps, void* workspace,
+                         size_t workspace_bytes, br_stream_t stream);
+
+/* ---- softmax family ---------------------------------------------------- */
+/* cudnnSoftmaxForward(ACCURATE, INSTANCE) at cuda_tensor.cpp:332-356 and
+ * cudnnSoftmaxBackward at :890-918.  y may alias x; dx may alias dy. */
+int br_hip_softmax_fwd(const float* x, float* y, int64_t rows, int64_t cols,
+                       br_stream_t stream);
+int br_hip_softmax_bwd(const float* dy, const float* y, float* dx, int64_t rows, int64_t cols,
+                       br_stream_t stream);
+
+/* The three-word sequence of bloomz-7b/train.words:158-162 in one pass:
+ * p = softmax((s + alibi[h,:]) + xmask[b,q,:]) over the last dimension of
+ * s[batch, heads, tq, tk], with alibi[heads, tk] and xmask[batch, tq, tk]
+ * (either may be NULL).  Same operation order as the separate ops, so the
+ * result is bit-identical to them.  p may alias s. */
+int br_hip_alibi_masked_softmax_fwd(const float* s, const float* alibi, const float* xmask,
+                                    float* p, int64_t batch, int64_t heads, int64_t tq,
+                                    int64_t tk, br_stream_t stream);
+
+/* The same, with the ALiBi bias and the causal / padding mask of
+ * blackriver/train_bloom.cpp:58-90 computed in the kernel from the device
+ * arrays slopes[heads] (fp64, as br_hip_alibi_slopes returns them) and
+ * valid[batch] (= number of leading non-zero mask entries per sequence)
+ * instead of being read from tables; bit-identical to the table form. */
+int br_hip_alibi_causal_softmax_fwd(const float* s, const double* slopes, const int32_t* valid,
+                                    float* p, int64_t batch, int64_t heads, int64_t tq,
+                                    int64_t tk, br_stream_t stream);
+
+/* cudnnSoftmaxForward(LOG) + kernels::nllloss_forward
+ * (kernels/nll_loss.cu:45-58, declared kernels/kernels.h:520) of cuda_tensor.cpp:535-553,640-652, one pass
+ * over logits[rows, vocab]:
+ *   lse[r]        = logsumexp(logits[r,:])
+ *   row_logp[r]   = keep[r] && 0 <= target[r] < vocab ?
+ *                   logits[r,target[r]] - lse[r] : 0
+ *   result[0]     = sum_r row_logp[r] / count   (+mean log-prob, the
+ *                   reference's sign convention, cuda_tensor.cpp:691)
+ *   result[1]     = count = #{r : keep[r] != 0}
+ * lse, row_logp: device fp32 [rows]; result: device fp32 [2]. */
+int br_hip_logsoftmax_nll_fwd(const float* logits, const int32_t* target, const int32_t* keep,
+                              float* lse, float* row_logp, float* result, int64_t rows,
+                              int64_t vocab, br_stream_t stream);
+
+/* cudnnSoftmaxBackward(LOG) of cuda_tensor.cpp:656-668 applied to the seed
+ * written by nll_loss.cu:33:
+ *   dlogits[r,c] = keep[r] ? (exp(logits[r,c]-lse[r]) - [c==target[r]])*scale : 0
+ * dlogits_dtype is BR_F32 or BR_F16; dlogits may alias logits when fp32. */
+int br_hip_logsoftmax_nll_bwd(const float* logits, const int32_t* target, const int32_t* keep,
+                              const float* lse, void* dlogits, int dlogits_dtype, float scale,
+                              int64_t rows, int64_t vocab, br_stream_t stream);
+
+/* ---- GEMM -------------------------------------------------------------- */
+enum {
+    BR_GEMM_F16 = 0,  /* operands rounded to fp16, v_mfma_f32_32x32x16_f16  */
+    BR_GEMM_BF16 = 1, /* operands rounded to bf16, v_mfma_f32_32x32x16_bf16 */
+    BR_GEMM_F32 = 2   /* fp32 operands, v_mfma_f32_32x32x2_f32              */
+};
+
+/* kernels::LtSgemm, kernels/LtSgemm.cu:55-126 (declared kernels/kernels.h:528-543),
+ * and the per-head loops around it at cuda_tensor.cpp:294-308,380-394 etc.
+ * Row-major, strided-batched, fp32 accumulation:
+ *
+ *   C[b][i,j] = alpha * sum_p opA[b][i,p] * opB[b][p,j]
+ *               + (accumulate ? C[b][i,j] : 0) + (bias ? bias[j] : 0)
+ *
+ *   trans_a == 0: A[b] is [m,k] with row stride lda;  1: A[b] is [k,m].
+ *   trans_b == 0: B[b] is [k,n] with row stride ldb;  1: B[b] is [n,k].
+ *
+ * a_dtype / b_dtype / c_dtype are BR_F32, BR_F16 or BR_BF16 storage types;
+ * `compute` picks the MFMA type operands are converted to on load.  stride_*
+ * are element strides between batch entries.  bias is fp32 [n] or NULL. */
+int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                const void* a, int a_dtype, int64_t lda, int64_t stride_a,
+                const void* b, int b_dtype, int64_t ldb, int64_t stride_b,
+                int accumulate, void* c, int c_dtype, int64_t ldc, int64_t stride_c,
+                const float* bias, int64_t batch, int compute, br_stream_t stream);
+
+/* ---- data preparation (bit-exact integer / gather work) ---------------- */
+/* The embedding row gather of blackriver/train_bloom.cpp:50-56. */
+int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, int elem_bytes,
+                            int64_t n, int64_t hidden, int64_t vocab, br_stream_t stream);
+/* The ALiBi table of train_bloom.cpp:58-71: alibi[h,k] = (float)(k*slope_h),
+ * slope_h = (2^(-2^(3-log2 heads)))^(h+1) evaluated in fp64 on the host. */
+int br_hip_alibi_table(float* alibi, int64_t heads, int64_t tokens, br_stream_t stream);
+/* The additive mask of train_bloom.cpp:73-90: xmask[b,q,k] = 0 when k <= q
+ * and mask[b,0..k] are all non-zero, else -FLT_MAX.  mask is device int32. */
+int br_hip_xmask_table(const int32_t* mask, float* xmask, int64_t batch, int64_t tokens,
+                       br_stream_t stream);
+/* Host helper: the fp64 ALiBi slopes of train_bloom.cpp:60-66. */
+int br_hip_alibi_slopes(double* slopes_host, int64_t heads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

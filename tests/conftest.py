@@ -38,3 +38,11 @@ def assert_close(got, ref, rtol, what=""):
     worst = float(np.max(err / bound)) if ref.size else 0.0
     assert worst <= 1.0, "%s: worst error %.3g x the %.1e bound (rms %.3g)" % (
         what, worst, rtol, rms)
+
+
+@pytest.fixture(autouse=True)
+def _release_device_temporaries(request):
+    yield
+    if request.node.get_closest_marker("gpu") is not None:
+        import gpu_util
+        gpu_util.release()

@@ -1,0 +1,184 @@
+"""Elementwise / data-movement HIP kernels against the CPU oracle through the
+C ABI: GELU and bias-GELU (fp32 and fp16 storage), broadcast add, transpose,
+column sums, casts and the bit-exact data-preparation tables."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from conftest import assert_close
+from gpu_util import (F16, F32, I32, assert_close_f16, call, dev, empty, host, ptr, stream, workspace)
+from blackriver_amd import hip
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+FLT_MAX = np.finfo(np.float32).max
+
+
+# ------------------------------------------------------------------- GELU
+@pytest.mark.parametrize("n", [8 * 1000, 1000003, 5])
+def test_gelu_f32_fwd_bwd(n):
+    rng = np.random.default_rng(0)
+    x = (1.5 * rng.standard_normal(n)).astype(np.float32)
+    x[:4] = [-12.0, 12.0, 0.0, -30.0][: min(4, n)]
+    dy = rng.standard_normal(n).astype(np.float32)
+    dx_, dy_ = dev(x), dev(dy)
+    y, g = empty(n), empty(n)
+    call("br_hip_gelu_fwd", ptr(dx_), ptr(y), F32, n, stream())
+    call("br_hip_gelu_bwd", ptr(dy_), ptr(dx_), ptr(g), F32, n, stream())
+    assert_close(host(y), orc.gelu_fwd(x), RTOL, "gelu fwd")
+    assert_close(host(g), orc.gelu_bwd(dy, x), RTOL, "gelu bwd")
+    # in place on x, the aliasing the scripts use (train.words:200)
+    call("br_hip_gelu_bwd", ptr(dy_), ptr(dx_), ptr(dx_), F32, n, stream())
+    assert np.array_equal(host(dx_), host(g))
+
+
+def test_bias_gelu_f16_headline_shape():
+    """x[2048,16384] fp16 ~N(0,1.5), bias ~N(0,0.02), dy ~N(0,1), seed 1."""
+    rng = np.random.default_rng(1)
+    rows, cols = 2048, 16384
+    x = (1.5 * rng.standard_normal((rows, cols))).astype(np.float16)
+    bias = (0.02 * rng.standard_normal(cols)).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float16)
+    dx_, db_, dy_ = dev(x), dev(bias), dev(dy)
+    y = empty((rows, cols), torch.float16)
+    g = empty((rows, cols), torch.float16)
+    dbias = empty(cols)
+    call("br_hip_bias_gelu_fwd", ptr(dx_), ptr(db_), ptr(y), F16, rows, cols, stream())
+    ws = workspace(hip.load().br_hip_bias_gelu_bwd_workspace(rows, cols))
+    call("br_hip_bias_gelu_bwd", ptr(dy_), ptr(dx_), ptr(db_), ptr(g), ptr(dbias), F16, rows, cols, ptr(ws),
+         ws.numel(), stream())
+    x32, dy32 = x.astype(np.float32), dy.astype(np.float32)
+    assert_close_f16(host(y), orc.bias_gelu_fwd(x32, bias), RTOL, "bias gelu fwd (fp16 storage)")
+    g_ref, _ = orc.bias_gelu_bwd(dy32, x32, bias)
+    got_g = host(g)
+    assert_close_f16(got_g, g_ref, RTOL, "bias gelu bwd (fp16 storage)")
+    # dbias sums what was stored (the fp16-rounded dx)
+    assert_close(host(dbias), got_g.astype(np.float64).sum(0), RTOL, "dbias")
+
+
+@pytest.mark.parametrize("rows,cols,dtype", [(33, 1024, "f32"), (7, 100, "f32"), (5, 24, "f16"), (9, 31, "f16")])
+def test_bias_gelu_small_and_unaligned(rows, cols, dtype):
+    rng = np.random.default_rng(2)
+    np_t, code, t_t = (np.float32, F32, torch.float32) if dtype == "f32" else (np.float16, F16, torch.float16)
+    x = (1.5 * rng.standard_normal((rows, cols))).astype(np_t)
+    bias = rng.standard_normal(cols).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np_t)
+    dx_, db_, dy_ = dev(x), dev(bias), dev(dy)
+    y, g, dbias = empty((rows, cols), t_t), empty((rows, cols), t_t), empty(cols)
+    call("br_hip_bias_gelu_fwd", ptr(dx_), ptr(db_), ptr(y), code, rows, cols, stream())
+    ws = workspace(hip.load().br_hip_bias_gelu_bwd_workspace(rows, cols))
+    call("br_hip_bias_gelu_bwd", ptr(dy_), ptr(dx_), ptr(db_), ptr(g), ptr(dbias), code, rows, cols, ptr(ws),
+         ws.numel(), stream())
+    y_ref = orc.bias_gelu_fwd(x.astype(np.float32), bias)
+    g_ref, dbias_ref = orc.bias_gelu_bwd(dy.astype(np.float32), x.astype(np.float32), bias)
+    if dtype == "f32":
+        assert_close(host(y), y_ref, RTOL, "fwd")
+        assert_close(host(g), g_ref, RTOL, "bwd")
+        assert_close(host(dbias), dbias_ref, RTOL, "dbias")
+    else:
+        assert_close_f16(host(y), y_ref, RTOL, "fwd")
+        assert_close_f16(host(g), g_ref, RTOL, "bwd")
+        assert_close(host(dbias), host(g).astype(np.float64).sum(0), RTOL, "dbias")
+
+
+# ---------------------------------------------------------- broadcast add
+@pytest.mark.parametrize("ashape,bshape", [
+    ((4, 32, 128, 128), (1, 32, 1, 128)),   # alibi
+    ((4, 32, 128, 128), (4, 1, 128, 128)),  # xmask
+    ((2, 512, 4096), (2, 512, 4096)),       # residual
+    ((2, 3, 5, 7), (1, 3, 1, 7)), ((2, 3, 5, 7), (2, 1, 5, 7)), ((6, 10), (1, 10)), ((2, 3, 4, 8), (2, 3, 4, 1)),
+])
+def test_add_bcast_bit_exact(ashape, bshape):
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal(ashape).astype(np.float32)
+    b = rng.standard_normal(bshape).astype(np.float32)
+    if bshape[-1] == ashape[-1] and len(bshape) == 4 and bshape[1] == 1:
+        b[b > 1.0] = -FLT_MAX          # behave like the additive mask
+    da, db_ = dev(a), dev(b)
+    c = empty(ashape)
+    call("br_hip_add_bcast", ptr(da), ptr(db_), ptr(c), F32, hip.shape4(ashape), hip.shape4(bshape), stream())
+    ref = orc.add_bcast(a, b)
+    assert np.array_equal(host(c), ref)
+    # c aliasing a (train.words:158)
+    call("br_hip_add_bcast", ptr(da), ptr(db_), ptr(da), F32, hip.shape4(ashape), hip.shape4(bshape), stream())
+    assert np.array_equal(host(da), ref)
+
+
+def test_add_f16_same_shape():
+    rng = np.random.default_rng(4)
+    a = rng.standard_normal((3, 40, 64)).astype(np.float16)
+    b = rng.standard_normal((3, 40, 64)).astype(np.float16)
+    c = empty(a.shape, torch.float16)
+    da, db_ = dev(a), dev(b)          # keep the operands alive until the kernel has run
+    call("br_hip_add_bcast", ptr(da), ptr(db_), ptr(c), F16, hip.shape4(a.shape), hip.shape4(b.shape), stream())
+    assert np.array_equal(host(c), (a.astype(np.float32) + b.astype(np.float32)).astype(np.float16))
+
+
+# ----------------------------------------------------- transpose / colsum
+@pytest.mark.parametrize("shape,eb", [((4, 512, 32, 128), 4), ((2, 7, 3, 5), 4), ((2, 16, 4, 8), 2), ((1, 3, 5, 3), 2)])
+def test_transpose_0213_bit_exact(shape, eb):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(shape).astype(np.float32 if eb == 4 else np.float16)
+    y = empty((shape[0], shape[2], shape[1], shape[3]), torch.float32 if eb == 4 else torch.float16)
+    call("br_hip_transpose_0213", ptr(dev(x)), ptr(y), eb, *shape, stream())
+    assert np.array_equal(host(y), np.ascontiguousarray(x.transpose(0, 2, 1, 3)))
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (77, 130), (1, 8)])
+def test_colsum(rows, cols):
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    out = empty(cols)
+    ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
+    call("br_hip_colsum", ptr(dev(x)), F32, ptr(out), rows, cols, ptr(ws), ws.numel(), stream())
+    assert_close(host(out), x.astype(np.float64).sum(0), RTOL, "colsum")
+
+
+def test_fill_and_cast_roundtrip():
+    n = 100003
+    t = empty(n)
+    call("br_hip_fill", ptr(t), F32, 2.5, n, stream())
+    assert np.all(host(t) == 2.5)
+    rng = np.random.default_rng(7)
+    x = (rng.standard_normal(n) * 10.0 ** rng.integers(-6, 5, n)).astype(np.float32)
+    h = empty(n, torch.float16)
+    call("br_hip_cast", ptr(dev(x)), F32, ptr(h), F16, n, stream())
+    with np.errstate(over="ignore"):
+        assert np.array_equal(host(h).view(np.uint16), x.astype(np.float16).view(np.uint16))
+    back = empty(n)
+    call("br_hip_cast", ptr(h), F16, ptr(back), F32, n, stream())
+    assert np.array_equal(host(back), host(h).astype(np.float32))
+
+
+# ------------------------------------------------ data preparation tables
+def test_embedding_gather_bit_exact(fixture_ids_mask):
+    ids, _ = fixture_ids_mask
+    rng = np.random.default_rng(8)
+    vocab, hidden = 4099, 4096
+    table = rng.standard_normal((vocab, hidden)).astype(np.float32)
+    small = (ids % vocab).astype(np.int32)
+    out = empty((2, 512, hidden))
+    call("br_hip_embedding_gather", ptr(dev(table)), ptr(dev(small)), ptr(out), 4, small.size, hidden, vocab, stream())
+    assert np.array_equal(host(out), orc.embedding_gather(table, small))
+
+
+@pytest.mark.parametrize("heads,tokens", [(32, 512), (8, 7), (160, 33)])
+def test_alibi_table_bit_exact(heads, tokens):
+    out = empty((heads, tokens))
+    call("br_hip_alibi_table", ptr(out), heads, tokens, stream())
+    assert np.array_equal(host(out), orc.alibi(heads, tokens))
+
+
+def test_xmask_table_bit_exact(fixture_ids_mask):
+    _, mask = fixture_ids_mask
+    m = mask.copy()
+    out = empty((2, 512, 512))
+    call("br_hip_xmask_table", ptr(dev(m)), ptr(out), 2, 512, stream())
+    assert np.array_equal(host(out), orc.xmask(m))
+    holes = np.array([[1, 1, 0, 1, 1], [0, 1, 1, 1, 1], [1, 1, 1, 1, 1]], np.int32)
+    out2 = empty((3, 5, 5))
+    call("br_hip_xmask_table", ptr(dev(holes)), ptr(out2), 3, 5, stream())
+    assert np.array_equal(host(out2), orc.xmask(holes))

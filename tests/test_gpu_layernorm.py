@@ -1,0 +1,101 @@
+"""LayerNorm forward / backward HIP kernels against the CPU oracle, through
+the C ABI.  Tolerance: 1e-5 relative (see conftest.assert_close), the bound
+stated for fp32 operators."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from conftest import assert_close
+from gpu_util import call, dev, empty, host, ptr, stream, workspace
+from blackriver_amd import hip
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+
+
+def run_fwd(x, g, b, eps, offset=0):
+    rows, cols = x.shape
+    if offset:   # place x at an address that is not 16-byte aligned
+        buf = empty(x.size + offset)
+        buf[offset:] = dev(x).flatten()
+        dx_ = buf[offset:]
+    else:
+        dx_ = dev(x)
+    y, mean, var = empty((rows, cols)), empty(rows), empty(rows)
+    dg, db = dev(g), dev(b)
+    call("br_hip_layernorm_fwd", ptr(dx_), ptr(dg), ptr(db), ptr(y), ptr(mean), ptr(var), rows, cols, eps, stream())
+    return host(y), host(mean), host(var)
+
+
+def run_bwd(dy, y, g, b, var, eps):
+    rows, cols = dy.shape
+    dgam, dbet, dx = empty(cols), empty(cols), empty((rows, cols))
+    ws = workspace(hip.load().br_hip_layernorm_bwd_workspace(rows, cols))
+    t = [dev(a) for a in (dy, y, g, b, var)]
+    call("br_hip_layernorm_bwd", ptr(t[0]), ptr(t[1]), ptr(t[2]), ptr(t[3]), ptr(t[4]), ptr(dgam), ptr(dbet),
+         ptr(dx), rows, cols, eps, ptr(ws), ws.numel(), stream())
+    return host(dx), host(dgam), host(dbet)
+
+
+def make(rows, cols, seed):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    g = (1 + 0.02 * rng.standard_normal(cols)).astype(np.float32)
+    b = (0.02 * rng.standard_normal(cols)).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    return x, g, b, dy
+
+
+@pytest.mark.parametrize("rows,cols", [
+    (2048, 4096),    # the headline configuration
+    (1, 4096), (3, 64), (37, 1024), (5, 8192), (7, 1000), (9, 1001), (4, 12), (2, 20000),
+])
+def test_layernorm_fwd_bwd_against_oracle(rows, cols):
+    print("case rows=%d cols=%d" % (rows, cols), flush=True)
+    x, g, b, dy = make(rows, cols, seed=0)
+    eps = 1e-5
+    y_ref, mean_ref, var_ref = orc.layernorm_fwd(x, g, b, eps)
+    y, mean, var = run_fwd(x, g, b, eps)
+    assert_close(y, y_ref, RTOL, "y")
+    assert_close(mean, mean_ref, RTOL, "mean")
+    assert_close(var, var_ref, RTOL, "var (sigma^2 + eps)")
+    # backward consumes the forward's own output and statistic, like the scripts do
+    dx_ref, dg_ref, db_ref = orc.layernorm_bwd(dy, y_ref, g, b, var_ref, eps)
+    dx, dg, db = run_bwd(dy, y_ref, g, b, var_ref, eps)
+    assert_close(dx, dx_ref, RTOL, "dx")
+    assert_close(dg, dg_ref, RTOL, "dgamma")
+    assert_close(db, db_ref, RTOL, "dbeta")
+
+
+def test_layernorm_unaligned_input_and_large_mean():
+    x, g, b, _ = make(6, 512, seed=1)
+    x = x * 0.1 + 50.0       # variance tiny next to the mean: needs the centred form
+    y_ref, _, var_ref = orc.layernorm_fwd(x, g, b, 1e-5)
+    y, _, var = run_fwd(x, g, b, 1e-5, offset=1)
+    assert_close(y, y_ref, 1e-4, "y, mean 50 / std 0.1")     # x itself carries 2^-24 * 50 / 0.1 of noise
+    assert_close(var, var_ref, 1e-4, "var")
+
+
+def test_layernorm_bwd_overwrites_grads_and_handles_tiny_gamma():
+    x, g, b, dy = make(16, 256, seed=2)
+    g[3], g[4] = 1e-7, -1e-7
+    eps = 1e-5
+    y_ref, _, var_ref = orc.layernorm_fwd(x, g, b, eps)
+    dx_ref, dg_ref, db_ref = orc.layernorm_bwd(dy, y_ref, g, b, var_ref, eps)
+    dx, dg, db = run_bwd(dy, y_ref, g, b, var_ref, eps)
+    assert_close(dx, dx_ref, RTOL, "dx")
+    assert_close(dg, dg_ref, RTOL, "dgamma with |gamma| < eps")
+    assert_close(db, db_ref, RTOL, "dbeta")
+
+
+def test_layernorm_rejects_bad_arguments():
+    lib = hip.load()
+    t = empty(16)
+    assert lib.br_hip_layernorm_fwd(None, ptr(t), ptr(t), ptr(t), None, None, 1, 16, 1e-5, stream()) == -2
+    assert lib.br_hip_layernorm_fwd(ptr(t), ptr(t), ptr(t), None, None, None, 1, 16, 1e-5, stream()) == -3
+    assert lib.br_hip_layernorm_fwd(ptr(t), ptr(t), ptr(t), ptr(t), None, None, 1, 0, 1e-5, stream()) == -4
+    assert lib.br_hip_layernorm_bwd(ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 1, 16, 1e-5,
+                                    None, 0, stream()) == -4
+    torch.cuda.synchronize()
