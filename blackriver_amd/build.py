@@ -31,7 +31,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-I" + INCLUDE, "-I" + HOST_DIR]
+CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-maybe-uninitialized", "-I" + INCLUDE, "-I" + HOST_DIR]
 
 
 def _run(cmd):
@@ -47,7 +47,16 @@ def _sources(folder, ext):
     return sorted(os.path.join(folder, f) for f in os.listdir(folder) if f.endswith(ext))
 
 
-def build_kernels(verbose=True):
+def _stale(obj, src, folder):
+    """True when obj is older than src or than any header next to it / in include/."""
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    deps = [src] + _sources(folder, ".hpp") + _sources(INCLUDE, ".h")
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build_kernels(verbose=True, force=True):
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)
     srcs = _sources(KERNEL_DIR, ".hip")
@@ -55,6 +64,8 @@ def build_kernels(verbose=True):
 
     def one(pair):
         src, obj = pair
+        if not force and not _stale(obj, src, KERNEL_DIR):
+            return ""
         return _run(["hipcc"] + HIPCC_FLAGS + ["-c", src, "-o", obj])
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
@@ -67,7 +78,7 @@ def build_kernels(verbose=True):
     return HIP_LIB
 
 
-def build_host(verbose=True):
+def build_host(verbose=True, force=True):
     srcs = _sources(HOST_DIR, ".cpp") if os.path.isdir(HOST_DIR) else []
     if not srcs:
         return None
@@ -77,6 +88,8 @@ def build_host(verbose=True):
 
     def one(pair):
         src, obj = pair
+        if not force and not _stale(obj, src, HOST_DIR):
+            return ""
         return _run(["g++"] + CXX_FLAGS + ["-c", src, "-o", obj])
 
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
@@ -90,11 +103,12 @@ def build_host(verbose=True):
     return HOST_LIB
 
 
-def build_all(verbose=True):
-    build_kernels(verbose)
-    build_host(verbose)
+def build_all(verbose=True, force=True):
+    build_kernels(verbose, force)
+    build_host(verbose, force)
 
 
 if __name__ == "__main__":
-    build_all()
+    # `--incremental` recompiles only sources that changed since the last build
+    build_all(force="--incremental" not in sys.argv)
     sys.exit(0)

@@ -1,0 +1,101 @@
+#include "bloom_input.hpp"
+
+#include <cfloat>
+#include <cmath>
+#include <cstring>
+
+#include "br_hip.h"
+#include "runtime.hpp"
+#include "tensor.hpp"
+
+namespace br {
+
+void BloomInput::gather_embeddings(const float* vocab, int64_t hidden, const int32_t* ids, int64_t n,
+                                   float* xinput) {
+    for (int64_t i = 0; i < n; i++)
+        memcpy(xinput + i * hidden, vocab + (int64_t)ids[i] * hidden, (size_t)hidden * sizeof(float));
+}
+
+void BloomInput::build_alibi(int64_t heads, int64_t tokens, float* alibi) {
+    std::vector<double> slopes((size_t)heads);
+    br_hip_alibi_slopes(slopes.data(), heads);  // pure host arithmetic
+    for (int64_t h = 0; h < heads; h++)
+        for (int64_t k = 0; k < tokens; k++) alibi[h * tokens + k] = (float)((double)k * 1.0 * slopes[(size_t)h]);
+}
+
+void BloomInput::build_xmask(const int32_t* mask, int64_t batch, int64_t tokens, float* xmask) {
+    for (int64_t b = 0; b < batch; b++) {
+        const int32_t* m = mask + b * tokens;
+        // number of leading real tokens: keys at or beyond it are closed for every query
+        int64_t open = 0;
+        while (open < tokens && m[open] != 0) open++;
+        float* plane = xmask + b * tokens * tokens;
+        for (int64_t q = 0; q < tokens; q++) {
+            const int64_t lim = q + 1 < open ? q + 1 : open;
+            float* row = plane + q * tokens;
+            for (int64_t k = 0; k < lim; k++) row[k] = 0.0f;
+            for (int64_t k = lim; k < tokens; k++) row[k] = -FLT_MAX;
+        }
+    }
+}
+
+namespace {
+
+struct Embed : public NativeWord {
+    void run(Stack& stack) override {
+        tensor_t out = stack.pop_tensor();
+        tensor_t table = stack.pop_tensor();
+        tensor_t ids = stack.pop_tensor();
+        br_assert(ids->is_cpu() && ids->dtype() == DataType::Int, "bloom.embed: ids must be a cpu int tensor");
+        br_assert(table->is_cuda() && out->is_cuda() && table->dtype() == out->dtype(),
+                  "bloom.embed: table and out must be device tensors of one type");
+        const int64_t hidden = (int64_t)table->shape().vec().back();
+        const int64_t vocab = (int64_t)table->items() / hidden;
+        const int64_t n = (int64_t)out->items() / hidden;
+        br_assert((int64_t)ids->items() >= n, "bloom.embed: not enough ids");
+        int32_t* d_ids = static_cast<int32_t*>(ComputingContext::scratch((size_t)n * sizeof(int32_t)));
+        BR_HIP_CHECK(br_hip_memcpy_h2d(d_ids, ids->data(), (size_t)n * sizeof(int32_t), ComputingContext::stream));
+        BR_HIP_CHECK(br_hip_embedding_gather(table->data(), d_ids, out->data(), (int)DataType_size(table->dtype()), n,
+                                             hidden, vocab, ComputingContext::stream));
+    }
+    NWORD_CREATOR_DEFINE_LR(Embed)
+};
+
+struct Alibi : public NativeWord {
+    void run(Stack& stack) override {
+        tensor_t alibi = stack.pop_tensor();
+        br_assert(alibi->is_cuda() && alibi->dtype() == DataType::Float && alibi->shape().dim() == 4,
+                  "bloom.alibi: expects a device fp32 tensor [1, heads, 1, tokens]");
+        BR_HIP_CHECK(br_hip_alibi_table(static_cast<float*>(alibi->data()), (int64_t)alibi->shape()[1],
+                                        (int64_t)alibi->shape()[3], ComputingContext::stream));
+    }
+    NWORD_CREATOR_DEFINE_LR(Alibi)
+};
+
+struct XMask : public NativeWord {
+    void run(Stack& stack) override {
+        tensor_t xmask = stack.pop_tensor();
+        tensor_t mask = stack.pop_tensor();
+        br_assert(mask->is_cpu() && mask->dtype() == DataType::Int, "bloom.xmask: mask must be a cpu int tensor");
+        br_assert(xmask->is_cuda() && xmask->dtype() == DataType::Float && xmask->shape().dim() == 4,
+                  "bloom.xmask: expects a device fp32 tensor [batch, 1, tokens, tokens]");
+        const int64_t batch = (int64_t)xmask->shape()[0], tokens = (int64_t)xmask->shape()[3];
+        br_assert((int64_t)mask->items() >= batch * tokens, "bloom.xmask: mask too small");
+        int32_t* d_mask = static_cast<int32_t*>(ComputingContext::scratch((size_t)(batch * tokens) * sizeof(int32_t)));
+        BR_HIP_CHECK(br_hip_memcpy_h2d(d_mask, mask->data(), (size_t)(batch * tokens) * sizeof(int32_t),
+                                       ComputingContext::stream));
+        BR_HIP_CHECK(br_hip_xmask_table(d_mask, static_cast<float*>(xmask->data()), batch, tokens,
+                                        ComputingContext::stream));
+    }
+    NWORD_CREATOR_DEFINE_LR(XMask)
+};
+
+}  // namespace
+
+void load_bloom_words(Enviroment& env) {
+    env.insert_native_word("bloom.embed", Embed::creator);
+    env.insert_native_word("bloom.alibi", Alibi::creator);
+    env.insert_native_word("bloom.xmask", XMask::creator);
+}
+
+}  // namespace br

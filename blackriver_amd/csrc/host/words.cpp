@@ -1,0 +1,173 @@
+// io.* / op.* word bindings.  Each word pops its operands from the stack,
+// last argument on top, and calls the TensorType operator of the same name;
+// the stack effects are those of the reference bindings
+// (blackriver/nn.cpp:16-337) so the model scripts run unchanged.
+#include "words.hpp"
+
+#include "br_hip.h"
+#include "runtime.hpp"
+#include "tensor.hpp"
+
+namespace br {
+
+namespace {
+
+std::vector<size_t> pop_shape(Stack& stack) {
+    std::vector<size_t> shape;
+    for (double d : stack.pop_number_list()) shape.push_back((size_t)d);
+    return shape;
+}
+
+// Pops N tensors; t[0] is the deepest (first pushed), t[N-1] was on top.
+template <size_t N>
+struct Tensors {
+    tensor_t t[N];
+    explicit Tensors(Stack& stack) {
+        for (size_t i = N; i-- > 0;) t[i] = stack.pop_tensor();
+    }
+    tensor_t& operator[](size_t i) { return t[i]; }
+};
+
+#define BR_WORD(CLS, ...)                                 \
+    struct CLS : public NativeWord {                      \
+        void run(Stack& stack) override { __VA_ARGS__ }   \
+        NWORD_CREATOR_DEFINE_LR(CLS)                      \
+    };
+
+// ( -- )  wait for everything queued on the compute stream
+BR_WORD(Sync, (void)stack; ComputingContext::sync();)
+
+// ( d0 .. dn-1 n device dtype -- tensor )
+BR_WORD(Create,
+    const std::string dtype = stack.pop_string();
+    const std::string device = stack.pop_string();
+    auto shape = pop_shape(stack);
+    tensor_t t;
+    if (device == "cuda" && dtype == "float") t = create_cuda_float(shape);
+    else if (device == "cuda" && dtype == "f16") t = create_cuda_f16(shape);
+    else if (device == "cuda" && dtype == "bf16") t = create_cuda_bf16(shape);
+    else if (device == "cpu" && dtype == "float") t = create_cpu_float(shape);
+    else if (device == "cpu" && dtype == "int") t = create_cpu_int(shape);
+    else br_panic("Can' be here!");
+    stack.push_tensor(t);
+)
+
+// ( "f32" | "f16" | "bf16" -- )  MFMA type for products whose operands are all
+// stored as fp32 (extension; fp32 is the default and matches the reference)
+BR_WORD(GemmPrecision,
+    const std::string p = stack.pop_string();
+    if (p == "f32" || p == "float") ComputingContext::fp32_gemm_compute = BR_GEMM_F32;
+    else if (p == "f16") ComputingContext::fp32_gemm_compute = BR_GEMM_F16;
+    else if (p == "bf16") ComputingContext::fp32_gemm_compute = BR_GEMM_BF16;
+    else br_panic("op.gemm_precision takes \"f32\", \"f16\" or \"bf16\"");
+)
+
+BR_WORD(Zero, tensor_t t = stack.pop_tensor(); t->op_zero(t);)
+// ( tensor value -- )
+BR_WORD(Fill, const double v = stack.pop_number(); tensor_t t = stack.pop_tensor(); t->op_fill(t, (float)v);)
+// ( tensor offset d0 .. dn-1 n -- view )
+BR_WORD(View,
+    auto shape = pop_shape(stack);
+    const size_t offset = (size_t)stack.pop_number();
+    tensor_t t = stack.pop_tensor();
+    auto ret = t->op_view(t, offset, shape);
+    stack.push_tensor(std::get<1>(ret));
+)
+// ( dst src -- )
+BR_WORD(Copy, Tensors<2> a(stack); a[0]->op_copy(a[0], a[1]);)
+// ( x w b y -- )
+BR_WORD(Linear, Tensors<4> a(stack); a[0]->op_linear(a[0], a[1], a[2], a[3]);)
+// ( x mean var scale bias y eps -- )
+BR_WORD(Layernorm,
+    const float eps = (float)stack.pop_number();
+    Tensors<6> a(stack);
+    a[0]->op_layernorm(a[0], a[1], a[2], a[3], a[4], a[5], eps);
+)
+// ( x y -- )
+BR_WORD(Transpos0213, Tensors<2> a(stack); a[0]->op_transpos_0213(a[0], a[1]);)
+// ( q k qk -- )
+BR_WORD(QueryKey, Tensors<3> a(stack); a[0]->op_qk(a[0], a[1], a[2]);)
+// ( a b c -- )
+BR_WORD(Add, Tensors<3> a(stack); a[0]->op_add(a[0], a[1], a[2]);)
+// ( x out -- )
+BR_WORD(Softmax, Tensors<2> a(stack); a[0]->op_softmax(a[0], a[1]);)
+// ( p v out -- )
+BR_WORD(Attn, Tensors<3> a(stack); a[0]->op_attn(a[0], a[1], a[2]);)
+// ( x out -- )
+BR_WORD(Gelu, Tensors<2> a(stack); a[0]->op_gelu(a[0], a[1]);)
+// ( x mask lm_head out -- )
+BR_WORD(LastLogits, Tensors<4> a(stack); a[0]->op_last_logits(a[0], a[1], a[2], a[3]);)
+// ( x ids mask lm_head workspace x_g lm_head_g -- )
+BR_WORD(LossBackward, Tensors<7> a(stack); a[0]->op_loss_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6]);)
+// ( dy scale bias var y dscale dbias din eps -- )
+BR_WORD(LayernormBackward,
+    const float eps = (float)stack.pop_number();
+    Tensors<8> a(stack);
+    a[0]->op_layernorm_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], eps);
+)
+// ( dy x w b x_g w_g b_g -- )
+BR_WORD(LinearBackward, Tensors<7> a(stack); a[0]->op_linear_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6]);)
+// ( dy x x_g -- )
+BR_WORD(GeluBackward, Tensors<3> a(stack); a[0]->op_gelu_backward(a[0], a[1], a[2]);)
+// ( dO attn v attn_g v_g -- )
+BR_WORD(AttnBackward, Tensors<5> a(stack); a[0]->op_attn_backward(a[0], a[1], a[2], a[3], a[4]);)
+// ( dy out x_g -- )
+BR_WORD(SoftmaxBackward, Tensors<3> a(stack); a[0]->op_softmax_backward(a[0], a[1], a[2]);)
+// ( dO attn v attn_g v_g -- )
+BR_WORD(SoftmaxAttnBackward, Tensors<5> a(stack); a[0]->op_softmax_attn_backward(a[0], a[1], a[2], a[3], a[4]);)
+// ( dS q k q_g k_g -- )
+BR_WORD(QueryKeyBackward, Tensors<5> a(stack); a[0]->op_qk_backward(a[0], a[1], a[2], a[3], a[4]);)
+
+BR_WORD(Dump, tensor_t t = stack.pop_tensor(); t->io_dump(t);)
+// ( tensor filename -- )
+BR_WORD(Load, const std::string f = stack.pop_string(); tensor_t t = stack.pop_tensor(); t->io_load(t, f.c_str());)
+BR_WORD(Save, const std::string f = stack.pop_string(); tensor_t t = stack.pop_tensor(); t->io_save(t, f.c_str());)
+// ( tensor peer -- )
+BR_WORD(MPIRecv, const int p = (int)stack.pop_number(); tensor_t t = stack.pop_tensor(); t->io_mpi_recv(t, p);)
+BR_WORD(MPIBcast, const int p = (int)stack.pop_number(); tensor_t t = stack.pop_tensor(); t->io_mpi_bcast(t, p);)
+BR_WORD(NcclRecv, const int p = (int)stack.pop_number(); tensor_t t = stack.pop_tensor(); t->io_nccl_recv(t, p);)
+BR_WORD(NcclSend, const int p = (int)stack.pop_number(); tensor_t t = stack.pop_tensor(); t->io_nccl_send(t, p);)
+
+}  // namespace
+
+void load_nn_words(Enviroment& env) {
+    static const struct {
+        const char* name;
+        NativeCreator* creator;
+    } table[] = {
+        {"io.dump", Dump::creator},
+        {"io.load", Load::creator},
+        {"io.save", Save::creator},
+        {"io.mpi.bcast", MPIBcast::creator},
+        {"io.mpi.recv", MPIRecv::creator},
+        {"io.nccl.send", NcclSend::creator},
+        {"io.nccl.recv", NcclRecv::creator},
+        {"op.sync", Sync::creator},
+        {"op.create", Create::creator},
+        {"op.gemm_precision", GemmPrecision::creator},
+        {"op.zero", Zero::creator},
+        {"op.fill", Fill::creator},
+        {"op.view", View::creator},
+        {"op.copy", Copy::creator},
+        {"op.linear", Linear::creator},
+        {"op.layernorm", Layernorm::creator},
+        {"op.transpos_0213", Transpos0213::creator},
+        {"op.add", Add::creator},
+        {"op.querykey", QueryKey::creator},
+        {"op.softmax", Softmax::creator},
+        {"op.attn", Attn::creator},
+        {"op.gelu", Gelu::creator},
+        {"op.last_logits", LastLogits::creator},
+        {"op.loss_backward", LossBackward::creator},
+        {"op.layernorm_backward", LayernormBackward::creator},
+        {"op.linear_backward", LinearBackward::creator},
+        {"op.gelu_backward", GeluBackward::creator},
+        {"op.attn_backward", AttnBackward::creator},
+        {"op.softmax_backward", SoftmaxBackward::creator},
+        {"op.softmax_attn_backward", SoftmaxAttnBackward::creator},
+        {"op.qk_backward", QueryKeyBackward::creator},
+    };
+    for (const auto& e : table) env.insert_native_word(e.name, e.creator);
+}
+
+}  // namespace br

@@ -1,0 +1,247 @@
+"""ctypes binding of ``libblackriver.so`` (the C embedding API declared in
+include/br_host.h): boot the C++ host runtime, run word scripts, move tensor
+contents.  Plumbing for drivers, tests and benchmarks written in Python; no
+fallback exists if the library has not been built.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libblackriver.so")
+WORDS_DIR = os.path.join(_PKG, "words")
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_cp = ctypes.c_char_p
+_dp = ctypes.POINTER(ctypes.c_double)
+_ip = ctypes.POINTER(_int)
+_f32p = ctypes.POINTER(ctypes.c_float)
+_i32p = ctypes.POINTER(ctypes.c_int32)
+
+SIGNATURES = {
+    "br_host_boot": (_int, [_int, ctypes.c_size_t]),
+    "br_host_shutdown": (_int, []),
+    "br_host_last_error": (_cp, []),
+    "br_host_stream": (_vp, []),
+    "br_host_sync": (_int, []),
+    "br_host_set_fp32_gemm_compute": (_int, [_int]),
+    "br_env_create": (_vp, [_int]),
+    "br_env_destroy": (None, [_vp]),
+    "br_env_execute": (_int, [_vp, _cp]),
+    "br_env_build": (_int, [_vp, _cp, _ip]),
+    "br_env_run": (_int, [_vp, _int]),
+    "br_env_change_hash": (_int, [_vp, _int]),
+    "br_env_current_hash": (_int, [_vp]),
+    "br_env_set_number": (_int, [_vp, _cp, ctypes.c_double]),
+    "br_env_set_string": (_int, [_vp, _cp, _cp]),
+    "br_env_get_number": (_int, [_vp, _cp, _dp]),
+    "br_env_has": (_int, [_vp, _cp]),
+    "br_env_stack_size": (_int, [_vp]),
+    "br_env_stack_clear": (_int, [_vp]),
+    "br_env_stack_pop_number": (_int, [_vp, _dp]),
+    "br_env_disassemble": (_int, [_vp, _cp, ctypes.c_char_p, ctypes.c_size_t]),
+    "br_env_tensor_info": (_int, [_vp, _cp, _ip, _ip, _ip, ctypes.POINTER(_i64), ctypes.POINTER(_vp)]),
+    "br_env_tensor_write": (_int, [_vp, _cp, _f32p, _i64]),
+    "br_env_tensor_read": (_int, [_vp, _cp, _f32p, _i64]),
+    "br_env_tensor_write_i32": (_int, [_vp, _cp, _i32p, _i64]),
+    "br_env_tensor_read_i32": (_int, [_vp, _cp, _i32p, _i64]),
+    "br_bloom_fetch_data": (_int, [_i32p, _i32p, _i64, _i64, _f32p, _i64, _i64, _f32p, _f32p, _f32p]),
+}
+
+_lib = None
+
+
+class HostError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HostError("%s is missing: build it with `python -m blackriver_amd.build`" % LIB_PATH)
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise HostError("%s: %s" % (what, load().br_host_last_error().decode(errors="replace")))
+
+
+_booted = False
+
+
+def boot(device: int = 0, host_arena_bytes: int = 1 << 30) -> None:
+    """Boot the runtime once per process (device < 0: host only)."""
+    global _booted
+    if _booted:
+        raise HostError("runtime already booted")
+    _check(load().br_host_boot(device, host_arena_bytes), "br_host_boot")
+    _booted = True
+
+
+def shutdown() -> None:
+    global _booted
+    if _booted:
+        _check(load().br_host_shutdown(), "br_host_shutdown")
+        _booted = False
+
+
+def booted() -> bool:
+    return _booted
+
+
+def stream():
+    return load().br_host_stream()
+
+
+def sync() -> None:
+    _check(load().br_host_sync(), "br_host_sync")
+
+
+def words_text(name: str) -> str:
+    """Text of one of the word scripts shipped with the package."""
+    with open(os.path.join(WORDS_DIR, name)) as f:
+        return f.read()
+
+
+class Env:
+    """An Enviroment with the io.*, op.* and bloom.* words loaded."""
+
+    def __init__(self, hashes: int = 1):
+        self._lib = load()
+        self._h = self._lib.br_env_create(hashes)
+        if not self._h:
+            raise HostError("br_env_create: " + self._lib.br_host_last_error().decode())
+
+    def close(self):
+        if self._h:
+            self._lib.br_env_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def execute(self, text: str) -> None:
+        rc = self._lib.br_env_execute(self._h, text.encode())
+        if rc != 0:
+            self._lib.br_env_stack_clear(self._h)
+        _check(rc, "execute")
+
+    def build(self, text: str) -> int:
+        prog = _int(-1)
+        _check(self._lib.br_env_build(self._h, text.encode(), ctypes.byref(prog)), "build")
+        return prog.value
+
+    def run(self, program: int) -> None:
+        _check(self._lib.br_env_run(self._h, program), "run")
+
+    def change_hash(self, h: int) -> None:
+        _check(self._lib.br_env_change_hash(self._h, h), "change_hash")
+
+    @property
+    def current_hash(self) -> int:
+        return self._lib.br_env_current_hash(self._h)
+
+    def set(self, name: str, value) -> None:
+        if isinstance(value, str):
+            _check(self._lib.br_env_set_string(self._h, name.encode(), value.encode()), "set")
+        else:
+            _check(self._lib.br_env_set_number(self._h, name.encode(), float(value)), "set")
+
+    def number(self, name: str) -> float:
+        v = ctypes.c_double()
+        _check(self._lib.br_env_get_number(self._h, name.encode(), ctypes.byref(v)), "number")
+        return v.value
+
+    def has(self, name: str) -> bool:
+        return bool(self._lib.br_env_has(self._h, name.encode()))
+
+    @property
+    def stack_size(self) -> int:
+        return self._lib.br_env_stack_size(self._h)
+
+    def stack_clear(self) -> None:
+        self._lib.br_env_stack_clear(self._h)
+
+    def pop_number(self) -> float:
+        v = ctypes.c_double()
+        _check(self._lib.br_env_stack_pop_number(self._h, ctypes.byref(v)), "pop_number")
+        return v.value
+
+    def disassemble(self, text: str) -> list:
+        """Compile and link `text`; return the flat step list as strings."""
+        size = 1 << 20
+        while True:
+            buf = ctypes.create_string_buffer(size)
+            rc = self._lib.br_env_disassemble(self._h, text.encode(), buf, size)
+            if rc == -2:
+                size *= 4
+                continue
+            _check(rc, "disassemble")
+            return buf.value.decode().split("\n")[:-1]
+
+    def info(self, name: str):
+        """(dtype code, on_device, shape tuple, data pointer) of a tensor."""
+        dtype, dev, rank = _int(), _int(), _int()
+        shape = (_i64 * 8)()
+        data = _vp()
+        _check(self._lib.br_env_tensor_info(self._h, name.encode(), ctypes.byref(dtype), ctypes.byref(dev),
+                                            ctypes.byref(rank), shape, ctypes.byref(data)), "info(%s)" % name)
+        return dtype.value, bool(dev.value), tuple(shape[i] for i in range(rank.value)), data.value
+
+    def write(self, name: str, array) -> None:
+        a = np.ascontiguousarray(array)
+        if a.dtype == np.int32:
+            _check(self._lib.br_env_tensor_write_i32(self._h, name.encode(), a.ctypes.data_as(_i32p), a.size),
+                   "write(%s)" % name)
+        else:
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            _check(self._lib.br_env_tensor_write(self._h, name.encode(), a.ctypes.data_as(_f32p), a.size),
+                   "write(%s)" % name)
+
+    def read(self, name: str) -> np.ndarray:
+        dtype, _, shape, _ = self.info(name)
+        if dtype == 3:
+            out = np.empty(shape, np.int32)
+            _check(self._lib.br_env_tensor_read_i32(self._h, name.encode(), out.ctypes.data_as(_i32p), out.size),
+                   "read(%s)" % name)
+        else:
+            out = np.empty(shape, np.float32)
+            _check(self._lib.br_env_tensor_read(self._h, name.encode(), out.ctypes.data_as(_f32p), out.size),
+                   "read(%s)" % name)
+        return out
+
+
+def fetch_data(ids, mask, heads, vocab=None):
+    """Host batch preparation: (xinput or None, alibi[heads,T], xmask[B,T,T])."""
+    ids = np.ascontiguousarray(ids, np.int32)
+    mask = np.ascontiguousarray(mask, np.int32)
+    b, t = ids.shape
+    alibi = np.empty((heads, t), np.float32)
+    xmask = np.empty((b, t, t), np.float32)
+    xinput = None
+    vp, hidden = None, 0
+    if vocab is not None:
+        vocab = np.ascontiguousarray(vocab, np.float32)
+        hidden = vocab.shape[1]
+        xinput = np.empty((b, t, hidden), np.float32)
+        vp = vocab.ctypes.data_as(_f32p)
+    _check(load().br_bloom_fetch_data(ids.ctypes.data_as(_i32p), mask.ctypes.data_as(_i32p), b, t, vp, hidden, heads,
+                                      xinput.ctypes.data_as(_f32p) if xinput is not None else None,
+                                      alibi.ctypes.data_as(_f32p), xmask.ctypes.data_as(_f32p)), "fetch_data")
+    return xinput, alibi, xmask

@@ -46,3 +46,14 @@ def _release_device_temporaries(request):
     if request.node.get_closest_marker("gpu") is not None:
         import gpu_util
         gpu_util.release()
+
+
+@pytest.fixture(scope="session")
+def runtime():
+    """Boots the C++ host runtime once per test process: on GPU 0 when one is
+    visible, host-only otherwise (creating a "cuda" tensor then panics)."""
+    import torch
+    from blackriver_amd import host
+    if not host.booted():
+        host.boot(0 if torch.cuda.is_available() else -1, 1 << 30)
+    return host

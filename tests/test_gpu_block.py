@@ -1,0 +1,214 @@
+"""The BLOOM block through the whole product path on the GPU: word script ->
+word machine -> TensorType -> HIPTensor -> br_hip kernels, compared buffer by
+buffer with the CPU oracle's composition of the same operator sequence.
+
+Two modes:
+  fp32   weights stored as fp32, products on the fp32 MFMA kernel
+         (bound 1e-4: a chain of ~20 fp32 operators, each within 1e-5)
+  f16    weights stored as fp16, every product on the fp16 MFMA kernel with
+         fp32 accumulation (bound 2e-2, the stated fp16-GEMM tolerance)
+"""
+import numpy as np
+import pytest
+
+import oracle as orc
+from oracle import bloom_block as blk
+from conftest import assert_close
+from blackriver_amd import host
+
+pytestmark = pytest.mark.gpu
+
+
+def setup_block(runtime, hidden, heads, batch, tokens, mode, vocab=1024, seed=3):
+    rng = np.random.default_rng(seed)
+    env = host.Env(2)
+    env.execute(host.words_text("bloom.words"))
+    env.execute("%d %d %d 1e-05 model_dims" % (hidden, heads, vocab))
+    env.set("$DEVICE", "cuda")
+    env.set("$WDTYPE", "f16" if mode == "f16" else "float")
+    env.execute("'%s' op.gemm_precision" % ("f16" if mode == "f16" else "f32"))
+    env.execute("create_layer_weight create_layer_grad zero_layer_grad")
+    env.execute("%d %d dynamic_floats" % (batch, tokens))
+    floats = int(env.pop_number()) + 64 * vocab
+    env.execute("%d create_var  %d %d create_dynamic" % (floats, batch, tokens))
+
+    w = blk.make_weights(rng, hidden, std=0.02)
+    if mode == "f16":   # the oracle sees the weights exactly as the device stores them
+        for k in w:
+            if k.endswith(".weight") and "layernorm" not in k:
+                w[k] = w[k].astype(np.float16).astype(np.float32)
+    env.write("query_key_value.weight", np.concatenate([w["query.weight"], w["key.weight"], w["value.weight"]]))
+    env.write("query_key_value.bias", np.concatenate([w["query.bias"], w["key.bias"], w["value.bias"]]))
+    for name in blk.WEIGHT_NAMES:
+        if not name.startswith(("query.", "key.", "value.")):
+            env.write(name, w[name])
+    x = rng.standard_normal((batch, tokens, hidden)).astype(np.float32)
+    dy = rng.standard_normal((batch, tokens, hidden)).astype(np.float32)
+    mask = np.ones((batch, tokens), np.int32)
+    mask[-1, tokens - tokens // 4:] = 0          # right padding on the last sequence
+    ids = rng.integers(0, vocab, (batch, tokens)).astype(np.int32)
+    env.write("mask_", mask)
+    env.write("ids_", ids)
+    env.write("xinput", x)
+    env.write("yout_g", dy)
+    env.execute("prepare_batch")
+    return env, w, x, dy, mask, ids
+
+
+@pytest.mark.parametrize("mode,hidden,heads,batch,tokens", [
+    ("fp32", 256, 4, 2, 24),
+    ("fp32", 1024, 8, 2, 128),
+    ("f16", 256, 4, 2, 24),
+    ("f16", 1024, 8, 2, 128),
+])
+def test_block_forward_backward_against_oracle(runtime, mode, hidden, heads, batch, tokens):
+    print("case", mode, hidden, heads, batch, tokens, flush=True)
+    tol = 1e-4 if mode == "fp32" else 2e-2
+    env, w, x, dy, mask, _ = setup_block(runtime, hidden, heads, batch, tokens, mode)
+    # the device-built tables are bit-exact
+    assert np.array_equal(env.read("alibi").reshape(heads, tokens), orc.alibi(heads, tokens))
+    assert np.array_equal(env.read("xmask").reshape(batch, tokens, tokens), orc.xmask(mask))
+
+    s = blk.layer_forward(w, x, orc.alibi(heads, tokens), orc.xmask(mask), heads)
+    env.execute("layer_forward op.sync")
+    for name in ("xattn_in", "zquery", "zkey", "zvalue", "xll", "xattn_out", "x4a", "x4b", "xa"):
+        assert_close(env.read(name).reshape(s[name].shape), s[name], tol, "forward " + name)
+    assert_close(env.read("input_ln_var")[: batch * tokens], s["input_ln_var"], tol, "input_ln_var")
+    assert_close(env.read("post_ln_var")[: batch * tokens], s["post_ln_var"], tol, "post_ln_var")
+
+    dx_ref, g_ref = blk.layer_backward(w, s, x, dy, heads)
+    env.execute("layer_backward_core op.sync")
+    assert_close(env.read("xa"), dx_ref, tol, "backward dx")
+    for name in blk.WEIGHT_NAMES:
+        if name == "key.bias":
+            continue
+        assert_close(env.read(name + "_g").reshape(g_ref[name + "_g"].shape), g_ref[name + "_g"], tol, name + "_g")
+    # key bias gradient is zero in exact arithmetic (softmax shift invariance)
+    scale = float(np.sqrt(np.mean(g_ref["query.bias_g"].astype(np.float64) ** 2)))
+    assert np.max(np.abs(env.read("key.bias_g"))) < (1e-3 if mode == "fp32" else 5e-2) * scale
+    env.close()
+
+
+def test_block_step_is_repeatable(runtime):
+    """Running the step twice from the same inputs gives the same bits: no
+    operator reads state it did not write in this step."""
+    env, w, x, dy, mask, _ = setup_block(runtime, 256, 4, 2, 24, "f16")
+    env.execute("block_step op.sync")
+    first = {n: env.read(n) for n in ("xa", "dense.weight_g", "query_key_value.weight_g", "input_layernorm.bias_g")}
+    env.write("yout_g", dy)       # layer_backward accumulates into yout_g in place
+    env.execute("block_step op.sync")
+    for n, v in first.items():
+        assert np.array_equal(env.read(n), v), n
+    env.close()
+
+
+@pytest.mark.parametrize("mode", ["fp32", "f16"])
+def test_loss_head_against_oracle(runtime, mode):
+    hidden, heads, batch, tokens, vocab = 256, 4, 2, 24, 1536
+    tol = 1e-4 if mode == "fp32" else 2e-2
+    env, _, x, _, mask, ids = setup_block(runtime, hidden, heads, batch, tokens, mode, vocab=vocab)
+    rng = np.random.default_rng(5)
+    lm = (0.05 * rng.standard_normal((vocab, hidden))).astype(np.float32)
+    if mode == "f16":
+        lm = lm.astype(np.float16).astype(np.float32)
+    g0 = rng.standard_normal((vocab, hidden)).astype(np.float32)
+    mask[0, 5] = 0                       # a hole: positions 4 and 5 carry no loss
+    env.write("mask_", mask)
+    env.execute("%d %d 2 'cuda' '%s' op.create 'lm_head.weight' !" % (vocab, hidden, "f16" if mode == "f16" else "float"))
+    env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight_g' !" % (vocab, hidden))
+    env.write("lm_head.weight", lm)
+    env.write("lm_head.weight_g", g0)
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xa' @ 'lm_head.weight_g' @ "
+                "op.loss_backward op.sync")
+    loss_ref, xg_ref, wg_ref, _ = orc.loss_backward(x, ids, mask, lm, lm_head_g=g0)
+    assert_close(env.read("xa"), xg_ref, tol, "x_g")
+    assert_close(env.read("lm_head.weight_g"), wg_ref, tol, "lm_head_g (accumulated)")
+    # a second call with a CPU gradient tensor, as the reference keeps it
+    env.execute("%d %d 2 'cpu' 'float' op.create 'lm_g_cpu' !  'lm_g_cpu' @ op.zero" % (vocab, hidden))
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xb' @ 'lm_g_cpu' @ op.loss_backward")
+    assert_close(env.read("lm_g_cpu"), wg_ref - g0, tol, "lm_head_g on the host")
+    assert np.array_equal(env.read("xb"), env.read("xa"))
+    env.close()
+
+
+def test_loss_value_and_chunking(runtime, capfd):
+    """The printed / returned value is +mean log-prob; a logits workspace that
+    holds only a few rows forces the chunked path."""
+    hidden, heads, batch, tokens, vocab = 256, 4, 2, 24, 512
+    env, _, x, _, mask, ids = setup_block(runtime, hidden, heads, batch, tokens, "fp32", vocab=vocab)
+    rng = np.random.default_rng(6)
+    lm = (0.05 * rng.standard_normal((vocab, hidden))).astype(np.float32)
+    env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight' !" % (vocab, hidden))
+    env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight_g' !  'lm_head.weight_g' @ op.zero" % (vocab, hidden))
+    env.write("lm_head.weight", lm)
+    env.execute("'all_logits' @ 0 7 %d 2 op.view 'few_rows' !" % vocab)       # room for 7 rows only
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'few_rows' @ 'xa' @ 'lm_head.weight_g' @ "
+                "op.loss_backward op.sync")
+    loss_ref, xg_ref, wg_ref, _ = orc.loss_backward(x, ids, mask, lm)
+    out = capfd.readouterr().out
+    line = [l for l in out.splitlines() if l.startswith("#################")][-1].split()
+    _, count = orc.loss_labels(ids, mask)
+    assert int(line[1]) == count
+    assert abs(float(line[2]) - loss_ref) <= 2e-5 * abs(loss_ref) + 1e-5
+    assert_close(env.read("xa"), xg_ref, 1e-4, "x_g (chunked)")
+    assert_close(env.read("lm_head.weight_g"), wg_ref, 1e-4, "lm_head_g (chunked)")
+    env.close()
+
+
+def test_unfused_attention_backward_and_last_logits(runtime):
+    hidden, heads, batch, tokens, vocab = 256, 4, 2, 24, 512
+    env, w, x, dy, mask, ids = setup_block(runtime, hidden, heads, batch, tokens, "fp32", vocab=vocab)
+    rng = np.random.default_rng(7)
+    hd = hidden // heads
+    p = orc.softmax_fwd(rng.standard_normal((batch, heads, tokens, tokens)).astype(np.float32))
+    v = rng.standard_normal((batch, heads, tokens, hd)).astype(np.float32)
+    d_o = rng.standard_normal((batch, heads, tokens, hd)).astype(np.float32)
+    env.write("xll", p)
+    env.write("zvalue", v)
+    env.write("zb", d_o)
+    env.execute("%d %d %d %d 4 'cuda' 'float' op.create 'dP' !" % (batch, heads, tokens, tokens))
+    env.execute("'zb' @ 'xll' @ 'zvalue' @ 'dP' @ 'za' @ op.attn_backward")
+    dp_ref, dv_ref = orc.attn_bwd(d_o, p, v)
+    assert_close(env.read("dP"), dp_ref, 1e-5, "dP")
+    assert_close(env.read("za"), dv_ref, 1e-5, "dV")
+    env.execute("'dP' @ 'xll' @ 'dP' @ op.softmax_backward")
+    assert_close(env.read("dP"), orc.softmax_bwd(dp_ref, p), 2e-5, "dS")
+
+    lm = (0.05 * rng.standard_normal((vocab, hidden))).astype(np.float32)
+    env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight' !" % (vocab, hidden))
+    env.execute("%d %d 2 'cuda' 'float' op.create 'last' !" % (batch, vocab))
+    env.write("lm_head.weight", lm)
+    env.execute("'xinput' @ 'mask_' @ 'lm_head.weight' @ 'last' @ op.last_logits")
+    assert_close(env.read("last"), orc.last_logits(x, mask, lm), 1e-5, "last logits")
+    env.close()
+
+
+def test_device_tensor_plumbing(runtime, tmp_path, capfd):
+    env = host.Env(1)
+    env.execute("2048 1 'cuda' 'float' op.create 'd' !  'd' @ 1.5 op.fill")
+    assert env.info("d")[1] and (env.read("d") == 1.5).all()
+    x = np.arange(2048, dtype=np.float32) / 7
+    f = tmp_path / "x.bin"
+    x.tofile(f)
+    env.execute("'d' @ '%s' io.load  'd' @ io.dump" % f)
+    assert np.array_equal(env.read("d"), x)
+    out = capfd.readouterr().out
+    assert "First 8 : 0 0.142857" in out and "Last 8 :" in out
+    # fp16 tensor: converted on load, on copy and on save
+    env.execute("2048 1 'cuda' 'f16' op.create 'h' !  'h' @ 'd' @ op.copy  'h' @ '%s' io.save" % (tmp_path / "h.bin"))
+    assert np.array_equal(np.fromfile(tmp_path / "h.bin", dtype=np.float32), x.astype(np.float16).astype(np.float32))
+    # host <-> device copies and views
+    env.execute("2048 1 'cpu' 'float' op.create 'c' !  'c' @ 'd' @ op.copy")
+    assert np.array_equal(env.read("c"), x)
+    env.execute("'d' @ op.zero  'd' @ 1024 2 512 2 op.view 'dv' !  'dv' @ 'c' @ 0 2 512 2 op.view op.copy")
+    got = env.read("d")
+    assert (got[:1024] == 0).all() and np.array_equal(got[1024:], x[:1024])
+    # in-process pipeline hand-off
+    env.execute("'d' @ 0 io.nccl.send  'd' @ op.zero  'd' @ 0 io.nccl.recv")
+    assert np.array_equal(env.read("d"), got)
+    with pytest.raises(host.HostError, match="nccl_recv"):
+        env.execute("'d' @ 1 io.nccl.recv")
+    # wrong size file
+    with pytest.raises(host.HostError, match="same size"):
+        env.execute("1024 1 'cuda' 'float' op.create '%s' io.load" % f)
+    env.close()
