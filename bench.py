@@ -1,0 +1,295 @@
+#!/usr/bin/env python3
+"""Benchmark of the BLOOM-7B1 training hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--leg all|block|roofline|elementwise]
+
+A "step" is one forward + backward pass of one BLOOM-7B1 decoder block
+(hidden 4096, 32 heads x 128, FFN 16384, ALiBi causal attention, batch 4 x
+seq 512, fp16 weights, fp32 activations and accumulation) run through the
+product path: word script -> word machine -> TensorType -> HIPTensor -> HIP
+kernels.  Inputs and weights are resident in HBM before the timed region.
+
+One JSON line is printed.  Besides the step throughput it carries
+  roofline      the dominant kernel (the MFMA GEMM at the h->4h shape of this
+                block) timed on its own with HIP events on the launch stream
+  elementwise   LayerNorm / bias-GELU / log-softmax+NLL kernels in GB/s
+  gemms         every GEMM shape of the block in TFLOP/s
+  cpu_baseline  the CPU oracle timed on the host cores on a bounded sample
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16
+
+H, NH, F, V = 4096, 32, 16384, 250880
+B, T = 4, 512
+N = B * T
+# GEMM flops of one block, forward (attention counted dense T x T)
+FWD_GEMM_FLOP = 2.0 * N * H * (3 * H + H + 2 * F) + 2 * 2.0 * B * NH * T * T * (H // NH)
+STEP_GEMM_FLOP = 3.0 * FWD_GEMM_FLOP
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--leg", default="all", choices=["all", "block", "roofline", "elementwise"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    return ap.parse_args()
+
+
+class Timer:
+    """HIP events recorded on the stream the kernels are launched on."""
+
+    def __init__(self, hip, stream):
+        self.hip, self.stream = hip, stream
+        self.device_sync = None
+        self.e0, self.e1 = ctypes.c_void_p(), ctypes.c_void_p()
+        hip.call("br_hip_event_create", ctypes.byref(self.e0))
+        hip.call("br_hip_event_create", ctypes.byref(self.e1))
+
+    def run(self, fn, iters, warmup):
+        if self.device_sync:
+            self.device_sync()   # buffers made on another stream are complete
+        for i in range(warmup):
+            fn(i)
+        self.hip.call("br_hip_stream_sync", self.stream)
+        self.hip.call("br_hip_event_record", self.e0, self.stream)
+        for i in range(iters):
+            fn(i)
+        self.hip.call("br_hip_event_record", self.e1, self.stream)
+        self.hip.call("br_hip_event_sync", self.e1)
+        ms = ctypes.c_float()
+        self.hip.call("br_hip_event_elapsed_ms", self.e0, self.e1, ctypes.byref(ms))
+        return ms.value * 1e-3 / iters   # seconds per iteration
+
+
+def block_leg(args, host, hip, timer):
+    rng = np.random.default_rng(3)
+    env = host.Env(2)
+    env.execute(host.words_text("bloom.words"))
+    env.execute("%d %d %d 1e-05 model_dims" % (H, NH, V))
+    env.set("$DEVICE", "cuda")
+    env.set("$WDTYPE", "f16")
+    env.execute("'f16' op.gemm_precision")
+    env.execute("create_layer_weight create_layer_grad zero_layer_grad")
+    env.execute("%d %d dynamic_floats" % (B, T))
+    floats = int(env.pop_number()) + V
+    env.execute("%d create_var  %d %d create_dynamic" % (floats, B, T))
+    env.execute("%d %d %d 3 'cuda' 'float' op.create 'yout_g0' !" % (B, T, H))
+
+    def normal(shape, std, mean=0.0):
+        return (mean + std * rng.standard_normal(shape)).astype(np.float32)
+
+    for ln in ("input_layernorm", "post_attention_layernorm"):
+        env.write(ln + ".weight", normal(H, 0.02, 1.0))
+        env.write(ln + ".bias", normal(H, 0.02))
+    for name, (o, i) in {"query_key_value": (3 * H, H), "dense": (H, H), "dense_h_to_4h": (F, H),
+                         "dense_4h_to_h": (H, F)}.items():
+        env.write(name + ".weight", normal((o, i), 0.02))
+        env.write(name + ".bias", normal(o, 0.02))
+    env.write("xinput", normal((B, T, H), 1.0))
+    env.write("yout_g0", normal((B, T, H), 1.0))
+    env.write("mask_", np.ones((B, T), np.int32))
+    env.execute("prepare_batch op.sync")
+    # the backward adds into yout_g in place, so every step starts from a fresh copy
+    step = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step")
+    sec = timer.run(lambda i: env.run(step), args.steps, args.warmup)
+    out = env.read("xa")
+    assert np.all(np.isfinite(out)), "block step produced non-finite values"
+    env.close()
+    return sec
+
+
+def gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch=1, iters=20):
+    tt = {hip.F32: torch.float32, hip.F16: torch.float16}
+    a = torch.randn((batch, m * k), device="cuda").to(tt[a_dt])
+    b = torch.randn((batch, n * k), device="cuda").to(tt[b_dt])
+    c = torch.empty((batch, m * n), device="cuda", dtype=tt[c_dt])
+    lda, ldb = (m if ta else k), (k if tb else n)
+    st = timer.stream
+
+    def fn(i):
+        hip.call("br_hip_gemm", ta, tb, m, n, k, 1.0, ctypes.c_void_p(a.data_ptr()), a_dt, lda, m * k,
+                 ctypes.c_void_p(b.data_ptr()), b_dt, ldb, n * k, 0, ctypes.c_void_p(c.data_ptr()), c_dt, n, m * n,
+                 None, batch, hip.GEMM_F16, st)
+    sec = timer.run(fn, iters, 3)
+    return sec, 2.0 * m * n * k * batch
+
+
+def roofline_leg(hip, timer, torch, full):
+    """Dominant kernel: the fp16 MFMA GEMM, activations fp32 x weights fp16,
+    at the h->4h shape [2048 x 4096] . [16384 x 4096]^T of this block."""
+    f32, f16 = hip.F32, hip.F16
+    sec, flop = gemm_case(hip, timer, torch, 0, 1, N, F, H, f32, f16, f32, iters=30)
+    roof = {"bound": "mfma", "kernel": "gemm_mfma16_kernel (A fp32 row-major, B fp16 [n,k], C fp32)",
+            "shape": "m=%d n=%d k=%d" % (N, F, H), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
+            "unit": "TFLOP/s", "frac": flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, "us_per_launch": sec * 1e6,
+            "traffic": None}
+    gemms = []
+    if full:
+        hd = H // NH
+        cases = [
+            ("qkv/dense fwd  y=xW^T", 0, 1, N, H, H, f32, f16, f32, 1),
+            ("h->4h fwd", 0, 1, N, F, H, f32, f16, f32, 1),
+            ("4h->h fwd", 0, 1, N, H, F, f32, f16, f32, 1),
+            ("dx=dy.W (4h->h)", 0, 0, N, F, H, f32, f16, f32, 1),
+            ("dx=dy.W (h->4h)", 0, 0, N, H, F, f32, f16, f32, 1),
+            ("dW=dy^T.x (h->4h)", 1, 0, F, H, N, f32, f32, f32, 1),
+            ("dW=dy^T.x (dense)", 1, 0, H, H, N, f32, f32, f32, 1),
+            ("QK^T", 0, 1, T, T, hd, f32, f32, f32, B * NH),
+            ("PV", 0, 0, T, hd, T, f32, f32, f32, B * NH),
+            ("dV=P^T.dO", 1, 0, T, hd, T, f32, f32, f32, B * NH),
+        ]
+        for name, ta, tb, m, n, k, a, b, c, batch in cases:
+            s, fl = gemm_case(hip, timer, torch, ta, tb, m, n, k, a, b, c, batch, iters=10)
+            gemms.append({"name": name, "m": m, "n": n, "k": k, "batch": batch, "us": round(s * 1e6, 1),
+                          "tflops": round(fl / s / 1e12, 1), "frac": round(fl / s / 1e12 / MFMA_F16_PEAK_TFLOPS, 3)})
+    return roof, gemms
+
+
+def elementwise_leg(hip, timer, torch):
+    """C1-C3 kernels; buffers are rotated so the 256 MB last-level cache
+    cannot serve the 33-134 MB working sets."""
+    lib = hip.load()
+    st = timer.stream
+    vp = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    out = {}
+
+    def rec(name, sec, nbytes):
+        gbs = nbytes / sec / 1e9
+        out[name] = {"us": round(sec * 1e6, 2), "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3),
+                     "algorithmic_MB": round(nbytes / 1e6, 2)}
+
+    nb = 8
+    rows, cols = 2048, 4096
+    xs = [torch.randn((rows, cols), device="cuda") for _ in range(nb)]
+    ys = [torch.empty_like(x) for x in xs]
+    dys = [torch.randn((rows, cols), device="cuda") for _ in range(nb)]
+    dxs = [torch.empty_like(x) for x in xs]
+    g = torch.randn(cols, device="cuda") * 0.02 + 1
+    b = torch.randn(cols, device="cuda") * 0.02
+    mean, var = torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda")
+    dg, db = torch.empty(cols, device="cuda"), torch.empty(cols, device="cuda")
+    sec = timer.run(lambda i: hip.call("br_hip_layernorm_fwd", vp(xs[i % nb]), vp(g), vp(b), vp(ys[i % nb]), vp(mean),
+                                       vp(var), rows, cols, 1e-5, st), 200, 10)
+    rec("layernorm_fwd [2048,4096] f32", sec, 2 * rows * cols * 4)
+    ws = torch.empty(lib.br_hip_layernorm_bwd_workspace(rows, cols), dtype=torch.uint8, device="cuda")
+    sec = timer.run(lambda i: hip.call("br_hip_layernorm_bwd", vp(dys[i % nb]), vp(ys[i % nb]), vp(g), vp(b), vp(var),
+                                       vp(dg), vp(db), vp(dxs[i % nb]), rows, cols, 1e-5, vp(ws), ws.numel(), st),
+                    200, 10)
+    rec("layernorm_bwd [2048,4096] f32", sec, 3 * rows * cols * 4)
+    del xs, ys, dys, dxs
+
+    rows, cols = 2048, 16384
+    xs = [(torch.randn((rows, cols), device="cuda") * 1.5).half() for _ in range(nb)]
+    ys = [torch.empty_like(x) for x in xs]
+    dys = [torch.randn((rows, cols), device="cuda").half() for _ in range(nb)]
+    bias = torch.randn(cols, device="cuda") * 0.02
+    dbias = torch.empty(cols, device="cuda")
+    sec = timer.run(lambda i: hip.call("br_hip_bias_gelu_fwd", vp(xs[i % nb]), vp(bias), vp(ys[i % nb]), hip.F16, rows,
+                                       cols, st), 200, 10)
+    rec("bias_gelu_fwd [2048,16384] f16", sec, 2 * rows * cols * 2)
+    ws = torch.empty(lib.br_hip_bias_gelu_bwd_workspace(rows, cols), dtype=torch.uint8, device="cuda")
+    sec = timer.run(lambda i: hip.call("br_hip_bias_gelu_bwd", vp(dys[i % nb]), vp(xs[i % nb]), vp(bias), vp(ys[i % nb]),
+                                       vp(dbias), hip.F16, rows, cols, vp(ws), ws.numel(), st), 200, 10)
+    rec("bias_gelu_bwd [2048,16384] f16 (+dbias)", sec, 3 * rows * cols * 2)
+    del xs, ys, dys
+
+    rows, vocab = 2048, V
+    logits = torch.randn((rows, vocab), device="cuda") * 2.0
+    dl = torch.empty_like(logits)
+    target = torch.randint(0, vocab, (rows,), device="cuda", dtype=torch.int32)
+    keep = (torch.rand(rows, device="cuda") < 0.9).to(torch.int32)
+    lse, rl, res = (torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda"), torch.empty(2, device="cuda"))
+    sec = timer.run(lambda i: hip.call("br_hip_logsoftmax_nll_fwd", vp(logits), vp(target), vp(keep), vp(lse), vp(rl),
+                                       vp(res), rows, vocab, st), 20, 3)
+    rec("logsoftmax_nll_fwd [2048,250880] f32", sec, rows * vocab * 4)
+    sec = timer.run(lambda i: hip.call("br_hip_logsoftmax_nll_bwd", vp(logits), vp(target), vp(keep), vp(lse), vp(dl),
+                                       hip.F32, 1.0 / rows, rows, vocab, st), 20, 3)
+    rec("logsoftmax_nll_bwd [2048,250880] f32", sec, 2 * rows * vocab * 4)
+    return out
+
+
+def cpu_baseline_leg():
+    """The CPU oracle (a restatement of the reference's operators; the
+    reference itself has no CPU math path) on a bounded sample: the same
+    block at batch 2 x 512 tokens, forward + backward, all host threads."""
+    import oracle as orc
+    from oracle import bloom_block as blk
+    rng = np.random.default_rng(3)
+    b, t = 2, 512
+    w = blk.make_weights(rng, H, std=0.02)
+    x = rng.standard_normal((b, t, H)).astype(np.float32)
+    dy = rng.standard_normal((b, t, H)).astype(np.float32)
+    alibi, xmask = orc.alibi(NH, t), orc.xmask(np.ones((b, t), np.int32))
+    t0 = time.perf_counter()
+    s = blk.layer_forward(w, x, alibi, xmask, NH)
+    blk.layer_backward(w, s, x, dy, NH)
+    sec = time.perf_counter() - t0
+    return {"value": b * t / sec, "unit": "tokens/s", "cores": orc.threads(), "kind": "port",
+            "sample": "same block (H=4096, 32 heads, FFN 16384) fwd+bwd at batch %d x %d tokens, fp32 storage with "
+                      "fp64 accumulation, %.1f s of CPU work" % (b, t, sec)}
+
+
+def main():
+    args = parse()
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        print("bench.py measures one GPU: every layer of a configuration lives on a single MI355X and there is no "
+              "multi-GPU path in this build (--gpus %d, WORLD_SIZE %d)." % (args.gpus, world), file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from blackriver_amd import hip, host
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.init()
+    host.boot(0, 1 << 30)
+    stream = ctypes.c_void_p(host.stream())
+    timer = Timer(hip, stream)
+    timer.device_sync = torch.cuda.synchronize
+
+    result = {"metric": "elementwise GB/s (% of 8 TB/s HBM) + BLOOM-7B1 block fwd+bwd tokens/sec",
+              "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+              "data": "synthetic",
+              "config": {"workload": "one BLOOM-7B1 decoder block fwd+bwd (BASELINE configs[3]): hidden 4096, "
+                                     "32 heads x 128, FFN 16384, ALiBi causal attention, batch 4 x seq 512, fp16 "
+                                     "weights ~N(0,0.02), fp32 activations and accumulation, seed 3",
+                         "tokens_per_step": N, "gemm_gflop_per_step": STEP_GEMM_FLOP / 1e9}}
+    if args.leg in ("all", "block"):
+        sec = block_leg(args, host, hip, timer)
+        result["value"] = N / sec
+        result["ms_per_step"] = sec * 1e3
+        result["step_gemm_tflops"] = STEP_GEMM_FLOP / sec / 1e12
+        result["step_frac_of_mfma_peak"] = STEP_GEMM_FLOP / sec / 1e12 / MFMA_F16_PEAK_TFLOPS
+    if args.leg in ("all", "roofline"):
+        roof, gemms = roofline_leg(hip, timer, torch, full=args.leg == "all")
+        result["roofline"] = roof
+        if gemms:
+            result["gemms"] = gemms
+    if args.leg in ("all", "elementwise"):
+        result["elementwise"] = elementwise_leg(hip, timer, torch)
+    if args.leg == "all" and not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline_leg()
+    host.sync()
+    print(json.dumps(result))
+    host.shutdown()
+
+
+if __name__ == "__main__":
+    main()
