@@ -60,6 +60,22 @@ constexpr size_t kTailBytes = 8u << 20;
 char* tail() { return static_cast<char*>(ComputingContext::workspace) + ComputingContext::workspace_size - kTailBytes; }
 size_t head_bytes() { return ComputingContext::workspace_size - kTailBytes; }
 
+// Every matrix product of the backend.  With a 16-bit MFMA type, fp32 operands
+// are staged as 16-bit copies first (br_hip_gemm_staged), which lets the
+// product run on the direct-to-LDS kernel; fp32 compute goes straight through.
+int product(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a, int a_dtype,
+            int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb, int64_t stride_b, int accumulate,
+            void* c, int c_dtype, int64_t ldc, int64_t stride_c, const float* bias, int64_t batch, int compute) {
+    void* stream = ComputingContext::stream;
+    if (compute == BR_GEMM_F32 || (a_dtype != BR_F32 && b_dtype != BR_F32))
+        return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
+                           accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
+    const size_t need = br_hip_gemm_staged_workspace(trans_a, trans_b, m, n, k, a_dtype, b_dtype, batch);
+    void* ws = ComputingContext::gemm_staging(need);
+    return br_hip_gemm_staged(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
+                              accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, ws, need, stream);
+}
+
 // fp32 device pointer to a bias vector, converting 16-bit storage on the fly
 // into workspace tail slot `slot` (each slot 1 MiB).
 const float* bias_f32(const tensor_t& b, int slot) {
@@ -240,8 +256,8 @@ ComputingReturn HIPTensor<DT>::op_linear(tensor_t self, tensor_t w, tensor_t bia
     if ((int64_t)w->shape()[1] != in || (int64_t)bias->items() != out) return OP_INPUT_ERROR;
     if ((int64_t)y->items() != n * out) return OP_OUTPUT_ERROR;
     // y[n,out] = x[n,in] . w[out,in]^T + bias, the bias added in the GEMM epilogue
-    BR_OP(br_hip_gemm(0, 1, n, out, in, 1.0f, mem_, (int)DT, in, 0, w->data(), code(w), in, 0, 0, y->data(), code(y),
-                      out, 0, bias_f32(bias, 0), 1, pick_compute({self, w, y}), stream()));
+    BR_OP(product(0, 1, n, out, in, 1.0f, mem_, (int)DT, in, 0, w->data(), code(w), in, 0, 0, y->data(), code(y),
+                      out, 0, bias_f32(bias, 0), 1, pick_compute({self, w, y})));
     return OP_OK;
 }
 
@@ -280,8 +296,8 @@ ComputingReturn HIPTensor<DT>::op_qk(tensor_t self, tensor_t k, tensor_t qk) {
     const int64_t bh = (int64_t)(s[0] * s[1]), t = (int64_t)s[2], hd = (int64_t)s[3];
     if (!dev(qk) || (int64_t)qk->items() != bh * t * t) return OP_OUTPUT_ERROR;
     const float alpha = (float)(1.0 / sqrt((double)hd));
-    BR_OP(br_hip_gemm(0, 1, t, t, hd, alpha, mem_, (int)DT, hd, t * hd, k->data(), code(k), hd, t * hd, 0, qk->data(),
-                      code(qk), t, t * t, nullptr, bh, pick_compute({self, k}), stream()));
+    BR_OP(product(0, 1, t, t, hd, alpha, mem_, (int)DT, hd, t * hd, k->data(), code(k), hd, t * hd, 0, qk->data(),
+                      code(qk), t, t * t, nullptr, bh, pick_compute({self, k})));
     return OP_OK;
 }
 
@@ -302,8 +318,8 @@ ComputingReturn HIPTensor<DT>::op_attn(tensor_t self, tensor_t v, tensor_t attn)
     const int64_t bh = (int64_t)(s[0] * s[1]), t = (int64_t)s[2], hd = (int64_t)v->shape()[3];
     if ((int64_t)v->items() != bh * t * hd) return OP_INPUT_ERROR;
     if (!dev(attn) || (int64_t)attn->items() != bh * t * hd) return OP_OUTPUT_ERROR;
-    BR_OP(br_hip_gemm(0, 0, t, hd, t, 1.0f, mem_, (int)DT, t, t * t, v->data(), code(v), hd, t * hd, 0, attn->data(),
-                      code(attn), hd, t * hd, nullptr, bh, pick_compute({self, v}), stream()));
+    BR_OP(product(0, 0, t, hd, t, 1.0f, mem_, (int)DT, t, t * t, v->data(), code(v), hd, t * hd, 0, attn->data(),
+                      code(attn), hd, t * hd, nullptr, bh, pick_compute({self, v})));
     return OP_OK;
 }
 
@@ -340,9 +356,8 @@ ComputingReturn HIPTensor<DT>::op_last_logits(tensor_t self, tensor_t mask_, ten
         BR_OP(br_hip_memcpy_d2d(rows + b * hidden, static_cast<const float*>(mem_) + (b * tokens + target) * hidden,
                                 hidden * sizeof(float), stream()));
     }
-    BR_OP(br_hip_gemm(0, 1, batch, vocab, hidden, 1.0f, rows, BR_F32, hidden, 0, lm_head->data(), code(lm_head),
-                      hidden, 0, 0, output->data(), BR_F32, vocab, 0, nullptr, 1, pick_compute({self, lm_head}),
-                      stream()));
+    BR_OP(product(0, 1, batch, vocab, hidden, 1.0f, rows, BR_F32, hidden, 0, lm_head->data(), code(lm_head),
+                      hidden, 0, 0, output->data(), BR_F32, vocab, 0, nullptr, 1, pick_compute({self, lm_head})));
     return OP_OK;
 }
 
@@ -424,16 +439,16 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
         bool any = false;
         for (int64_t r = r0; r < r0 + rows; r++) any = any || keep[r] != 0;
         if (!any) continue;  // nothing but zero gradients in this chunk
-        BR_OP(br_hip_gemm(0, 1, rows, vocab, hidden, 1.0f, x + r0 * hidden, BR_F32, hidden, 0, lm_head->data(),
-                          code(lm_head), hidden, 0, 0, logits, BR_F32, vocab, 0, nullptr, 1, compute, stream()));
+        BR_OP(product(0, 1, rows, vocab, hidden, 1.0f, x + r0 * hidden, BR_F32, hidden, 0, lm_head->data(),
+                          code(lm_head), hidden, 0, 0, logits, BR_F32, vocab, 0, nullptr, 1, compute));
         BR_OP(br_hip_logsoftmax_nll_fwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, d_logp + r0, d_result, rows,
                                         vocab, stream()));
         BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, logits, BR_F32, scale, rows,
                                         vocab, stream()));
-        BR_OP(br_hip_gemm(0, 0, rows, hidden, vocab, 1.0f, logits, BR_F32, vocab, 0, lm_head->data(), code(lm_head),
-                          hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute, stream()));
-        BR_OP(br_hip_gemm(1, 0, vocab, hidden, rows, 1.0f, logits, BR_F32, vocab, 0, x + r0 * hidden, BR_F32, hidden,
-                          0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute, stream()));
+        BR_OP(product(0, 0, rows, hidden, vocab, 1.0f, logits, BR_F32, vocab, 0, lm_head->data(), code(lm_head),
+                          hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute));
+        BR_OP(product(1, 0, vocab, hidden, rows, 1.0f, logits, BR_F32, vocab, 0, x + r0 * hidden, BR_F32, hidden,
+                          0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
     }
 
     // sum of log p(label) in fp64 on the host, as the reference accumulates it
@@ -504,11 +519,11 @@ ComputingReturn HIPTensor<DT>::op_linear_backward(tensor_t self, tensor_t x, ten
     void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
     BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, ws, need, stream()));
     // weight_g[out,in] = dy^T . x
-    BR_OP(br_hip_gemm(1, 0, out, in, n, 1.0f, mem_, (int)DT, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
-                      code(weight_g), in, 0, nullptr, 1, compute, stream()));
+    BR_OP(product(1, 0, out, in, n, 1.0f, mem_, (int)DT, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
+                      code(weight_g), in, 0, nullptr, 1, compute));
     // x_g[n,in] = dy . W
-    BR_OP(br_hip_gemm(0, 0, n, in, out, 1.0f, mem_, (int)DT, out, 0, weight->data(), code(weight), in, 0, 0,
-                      x_g->data(), code(x_g), in, 0, nullptr, 1, compute, stream()));
+    BR_OP(product(0, 0, n, in, out, 1.0f, mem_, (int)DT, out, 0, weight->data(), code(weight), in, 0, 0,
+                      x_g->data(), code(x_g), in, 0, nullptr, 1, compute));
     return OP_OK;
 }
 
@@ -544,10 +559,10 @@ ComputingReturn HIPTensor<DT>::op_attn_backward(tensor_t self, tensor_t attn, te
     if (!dev(attn_g) || !dev(v_g) || attn_g->items() != attn->items() || v_g->items() != v->items())
         return OP_OUTPUT_ERROR;
     const int compute = pick_compute({self, attn, v});
-    BR_OP(br_hip_gemm(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, mem_, (int)DT, d.hd,
-                      d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute, stream()));
-    BR_OP(br_hip_gemm(0, 1, d.t, d.t, d.hd, 1.0f, mem_, (int)DT, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
-                      d.t * d.hd, 0, attn_g->data(), code(attn_g), d.t, d.t * d.t, nullptr, d.bh, compute, stream()));
+    BR_OP(product(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, mem_, (int)DT, d.hd,
+                      d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute));
+    BR_OP(product(0, 1, d.t, d.t, d.hd, 1.0f, mem_, (int)DT, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
+                      d.t * d.hd, 0, attn_g->data(), code(attn_g), d.t, d.t * d.t, nullptr, d.bh, compute));
     return OP_OK;
 }
 
@@ -573,11 +588,11 @@ ComputingReturn HIPTensor<DT>::op_softmax_attn_backward(tensor_t self, tensor_t 
     if (!dev_f32(attn_g) || !dev(v_g) || attn_g->items() != attn->items() || v_g->items() != v->items())
         return OP_OUTPUT_ERROR;
     const int compute = pick_compute({self, attn, v});
-    BR_OP(br_hip_gemm(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, mem_, (int)DT, d.hd,
-                      d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute, stream()));
+    BR_OP(product(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, mem_, (int)DT, d.hd,
+                      d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute));
     float* dp = static_cast<float*>(ComputingContext::scratch((size_t)(d.bh * d.t * d.t) * sizeof(float)));
-    BR_OP(br_hip_gemm(0, 1, d.t, d.t, d.hd, 1.0f, mem_, (int)DT, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
-                      d.t * d.hd, 0, dp, BR_F32, d.t, d.t * d.t, nullptr, d.bh, compute, stream()));
+    BR_OP(product(0, 1, d.t, d.t, d.hd, 1.0f, mem_, (int)DT, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
+                      d.t * d.hd, 0, dp, BR_F32, d.t, d.t * d.t, nullptr, d.bh, compute));
     BR_OP(br_hip_softmax_bwd(dp, static_cast<const float*>(attn->data()), static_cast<float*>(attn_g->data()),
                              d.bh * d.t, d.t, stream()));
     return OP_OK;
@@ -593,10 +608,10 @@ ComputingReturn HIPTensor<DT>::op_qk_backward(tensor_t self, tensor_t q, tensor_
     if (!dev(q_g) || !dev(k_g) || q_g->items() != q->items() || k_g->items() != q->items()) return OP_OUTPUT_ERROR;
     const float alpha = (float)(1.0 / sqrt((double)hd));
     const int compute = pick_compute({self, q, k});
-    BR_OP(br_hip_gemm(0, 0, t, hd, t, alpha, mem_, (int)DT, t, t * t, k->data(), code(k), hd, t * hd, 0, q_g->data(),
-                      code(q_g), hd, t * hd, nullptr, bh, compute, stream()));
-    BR_OP(br_hip_gemm(1, 0, t, hd, t, alpha, mem_, (int)DT, t, t * t, q->data(), code(q), hd, t * hd, 0, k_g->data(),
-                      code(k_g), hd, t * hd, nullptr, bh, compute, stream()));
+    BR_OP(product(0, 0, t, hd, t, alpha, mem_, (int)DT, t, t * t, k->data(), code(k), hd, t * hd, 0, q_g->data(),
+                      code(q_g), hd, t * hd, nullptr, bh, compute));
+    BR_OP(product(1, 0, t, hd, t, alpha, mem_, (int)DT, t, t * t, q->data(), code(q), hd, t * hd, 0, k_g->data(),
+                      code(k_g), hd, t * hd, nullptr, bh, compute));
     return OP_OK;
 }
 

@@ -54,6 +54,8 @@ size_t ComputingContext::workspace_size = 0;
 int ComputingContext::fp32_gemm_compute = BR_GEMM_F32;
 void* ComputingContext::scratch_ptr_ = nullptr;
 size_t ComputingContext::scratch_size_ = 0;
+void* ComputingContext::staging_ptr_ = nullptr;
+size_t ComputingContext::staging_size_ = 0;
 
 void ComputingContext::boot(int dev) {
     br_assert(device < 0, "ComputingContext is already booted");
@@ -71,10 +73,11 @@ void ComputingContext::shutdown() {
     sync();
     free(host_workspace);
     if (scratch_ptr_) BR_HIP_CHECK(br_hip_free(scratch_ptr_));
+    if (staging_ptr_) BR_HIP_CHECK(br_hip_free(staging_ptr_));
     BR_HIP_CHECK(br_hip_free(workspace));
     BR_HIP_CHECK(br_hip_stream_destroy(stream));
-    host_workspace = workspace = stream = scratch_ptr_ = nullptr;
-    workspace_size = scratch_size_ = 0;
+    host_workspace = workspace = stream = scratch_ptr_ = staging_ptr_ = nullptr;
+    workspace_size = scratch_size_ = staging_size_ = 0;
     device = -1;
 }
 
@@ -94,6 +97,19 @@ void* ComputingContext::scratch(size_t bytes) {
         scratch_size_ = bytes;
     }
     return scratch_ptr_;
+}
+
+void* ComputingContext::gemm_staging(size_t bytes) {
+    br_assert(device >= 0, "ComputingContext is not booted");
+    if (bytes > staging_size_) {
+        sync();
+        if (staging_ptr_) BR_HIP_CHECK(br_hip_free(staging_ptr_));
+        // room to spare, so that a slightly larger product does not reallocate
+        bytes += bytes / 4;
+        BR_HIP_CHECK(br_hip_malloc(&staging_ptr_, bytes));
+        staging_size_ = bytes;
+    }
+    return staging_ptr_;
 }
 
 // ----------------------------------------------------- CollectiveContext

@@ -33,10 +33,15 @@ struct ComputingContext {
     // Grow-only device scratch for operators whose need exceeds `workspace`
     // (the attention backward stages dP for all heads at once).
     static void* scratch(size_t bytes);
+    // Grow-only device block of its own for the 16-bit operand copies the
+    // GEMM entry point stages (never the workspace: operands may live there).
+    static void* gemm_staging(size_t bytes);
 
 private:
     static void* scratch_ptr_;
     static size_t scratch_size_;
+    static void* staging_ptr_;
+    static size_t staging_size_;
 };
 
 // One process, one GPU: rank 0 of a world of 1.  `now()` keeps feeding the

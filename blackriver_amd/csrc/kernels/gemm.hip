@@ -3,11 +3,14 @@
 //   C[b][i,j] = alpha * sum_p opA[b][i,p] * opB[b][p,j] (+ C) (+ bias[j])
 //
 // 16-bit multiplicands (fp16 / bf16, fp32 accumulation) go to the kernel
-// template in gemm_mfma16.hpp; this file holds the argument checking, the
-// choice of tile configuration and the kernel that keeps fp32 operands and
+// templates in gemm_dtl16.hpp (both operands stored in the MFMA type, aligned:
+// direct-to-LDS loads) and gemm_mfma16.hpp (everything else: fp32 operands
+// converted on load, ragged sizes).  This file holds the argument checking,
+// the staging of fp32 operands into a caller's workspace so that they too can
+// take the direct-to-LDS kernel, and the kernel that keeps fp32 operands and
 // multiplies with v_mfma_f32_32x32x2_f32 for callers that need fp32-faithful
-// products (128x128x16 tiles, 4 wave64s x 2x2 MFMA blocks, same register
-// prefetch + LDS double buffering).
+// products (128x128x16 tiles, 4 wave64s x 2x2 MFMA blocks, register prefetch +
+// LDS double buffering).
 #include "common.hpp"
 
 #include <hip/hip_bf16.h>
@@ -244,16 +247,126 @@ extern "C" int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64
     p.a_kstr = ak;
     p.b_kstr = bk;
     p.c_dtype = c_dtype;
-    // 256x128 tiles once there are enough of them to fill the 256 CUs and K is
-    // long enough to amortise the larger prologue; BR_GEMM_TILE=big|small overrides
-    const long long big_blocks = ((m + 255) / 256) * ((n + 127) / 128) * batch;
-    p.big = m >= 256 && k >= 256 && big_blocks >= 192;
     // the fast kernel loads 128 bits at a time and never checks k
     const long long va = p.a_f32 ? 4 : 8, vb = p.b_f32 ? 4 : 8;
     p.guarded = !g.vec_a || !g.vec_b || k % 32 != 0 || (ak && m % va != 0) || (bk && n % vb != 0);
-    static const char* force = getenv("BR_GEMM_TILE");
-    if (force && strcmp(force, "big") == 0) p.big = true;
-    if (force && strcmp(force, "small") == 0) p.big = false;
     if (compute == BR_GEMM_F16) return gemm16_launch_f16(g, p, batch, st);
     return gemm16_launch_bf16(g, p, batch, st);
+}
+
+// ---- fp32 operands staged as 16-bit copies ----------------------------------
+namespace {
+
+// dst[b][r][c] (dense) = convert(src[b*stride + r*ld + c]); cols % 4 == 0 and
+// 16-byte aligned rows take the vector path.
+template <typename DST, bool VEC>
+__global__ __launch_bounds__(256) void stage_rows_kernel(const float* __restrict__ src, long long ld,
+                                                         long long stride, long long rows, long long cols,
+                                                         long long batch, DST* __restrict__ dst) {
+    const long long per_row = VEC ? cols / 4 : cols;
+    const long long total = batch * rows * per_row;
+    for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < total;
+         i += (long long)gridDim.x * blockDim.x) {
+        const long long c = i % per_row, r = (i / per_row) % rows, b = i / (per_row * rows);
+        const float* s = src + b * stride + r * ld;
+        DST* d = dst + (b * rows + r) * cols;
+        if (VEC) {
+            const float4 v = reinterpret_cast<const float4*>(s)[c];
+            gemm16::u32x2 o;
+            if (sizeof(DST) == 2 && __is_same(DST, __half)) {
+                o.x = gemm16::pack2(gemm16::Cvt<BR_GEMM_F16>::from_f32(v.x), gemm16::Cvt<BR_GEMM_F16>::from_f32(v.y));
+                o.y = gemm16::pack2(gemm16::Cvt<BR_GEMM_F16>::from_f32(v.z), gemm16::Cvt<BR_GEMM_F16>::from_f32(v.w));
+            } else {
+                o.x = gemm16::pack2(gemm16::Cvt<BR_GEMM_BF16>::from_f32(v.x), gemm16::Cvt<BR_GEMM_BF16>::from_f32(v.y));
+                o.y = gemm16::pack2(gemm16::Cvt<BR_GEMM_BF16>::from_f32(v.z), gemm16::Cvt<BR_GEMM_BF16>::from_f32(v.w));
+            }
+            reinterpret_cast<gemm16::u32x2*>(d)[c] = o;
+        } else {
+            const unsigned short h = __is_same(DST, __half) ? gemm16::Cvt<BR_GEMM_F16>::from_f32(s[c])
+                                                            : gemm16::Cvt<BR_GEMM_BF16>::from_f32(s[c]);
+            reinterpret_cast<unsigned short*>(d)[c] = h;
+        }
+    }
+}
+
+int stage_rows(const float* src, long long ld, long long stride, long long rows, long long cols, long long batch,
+               void* dst, int compute, hipStream_t st) {
+    const bool vec = cols % 4 == 0 && ld % 4 == 0 && stride % 4 == 0 && aligned16(src) && aligned16(dst);
+    const long long work = batch * rows * (vec ? cols / 4 : cols);
+    const unsigned grid = grid_for(work, 256, 1 << 16);
+    if (compute == BR_GEMM_F16) {
+        if (vec) stage_rows_kernel<__half, true><<<grid, 256, 0, st>>>(src, ld, stride, rows, cols, batch, (__half*)dst);
+        else stage_rows_kernel<__half, false><<<grid, 256, 0, st>>>(src, ld, stride, rows, cols, batch, (__half*)dst);
+    } else {
+        if (vec) stage_rows_kernel<__hip_bfloat16, true><<<grid, 256, 0, st>>>(src, ld, stride, rows, cols, batch, (__hip_bfloat16*)dst);
+        else stage_rows_kernel<__hip_bfloat16, false><<<grid, 256, 0, st>>>(src, ld, stride, rows, cols, batch, (__hip_bfloat16*)dst);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+size_t staged_bytes(int64_t rows, int64_t cols, int64_t batch) {
+    const size_t b = (size_t)rows * (size_t)cols * (size_t)batch * 2;
+    return (b + 255) & ~(size_t)255;
+}
+
+}  // namespace
+
+extern "C" size_t br_hip_gemm_staged_workspace(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, int a_dtype,
+                                               int b_dtype, int64_t batch) {
+    (void)trans_a;
+    (void)trans_b;
+    if (m <= 0 || n <= 0 || k <= 0 || batch <= 0) return 0;
+    size_t need = 0;
+    if (a_dtype == BR_F32) need += staged_bytes(m, k, batch);
+    if (b_dtype == BR_F32) need += staged_bytes(k, n, batch);
+    return need;
+}
+
+extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
+                                  int a_dtype, int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb,
+                                  int64_t stride_b, int accumulate, void* c, int c_dtype, int64_t ldc,
+                                  int64_t stride_c, const float* bias, int64_t batch, int compute, void* workspace,
+                                  size_t workspace_bytes, br_stream_t stream) {
+    const bool f32_a = a_dtype == BR_F32, f32_b = b_dtype == BR_F32;
+    const bool sixteen = compute == BR_GEMM_F16 || compute == BR_GEMM_BF16;
+    // Stage only when the converted problem meets the direct-to-LDS kernel's
+    // rules; every other case is the plain entry point's business.
+    const int64_t a_rows = trans_a ? k : m, a_cols = trans_a ? m : k;
+    const int64_t b_rows = trans_b ? n : k, b_cols = trans_b ? k : n;
+    bool stage = sixteen && (f32_a || f32_b) && workspace && aligned16(workspace) && m > 0 && n > 0 && k > 0 &&
+                 batch > 0 && a && b && k % 32 == 0;
+    if (stage) {
+        // dense 16-bit copies: leading dimension = cols, batch stride = rows*cols
+        if (f32_a && a_cols % 8 != 0) stage = false;
+        if (f32_b && b_cols % 8 != 0) stage = false;
+        if (lda < a_cols || ldb < b_cols) stage = false;
+        if (br_hip_gemm_staged_workspace(trans_a, trans_b, m, n, k, a_dtype, b_dtype, batch) > workspace_bytes)
+            stage = false;
+    }
+    if (!stage)
+        return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
+                           accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
+    const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
+    hipStream_t st = as_stream(stream);
+    char* ws = static_cast<char*>(workspace);
+    if (f32_a) {
+        const int rc = stage_rows(static_cast<const float*>(a), lda, stride_a, a_rows, a_cols, batch, ws, compute, st);
+        if (rc != BR_OK) return rc;
+        a = ws;
+        a_dtype = native;
+        lda = a_cols;
+        stride_a = a_rows * a_cols;
+        ws += staged_bytes(m, k, batch);
+    }
+    if (f32_b) {
+        const int rc = stage_rows(static_cast<const float*>(b), ldb, stride_b, b_rows, b_cols, batch, ws, compute, st);
+        if (rc != BR_OK) return rc;
+        b = ws;
+        b_dtype = native;
+        ldb = b_cols;
+        stride_b = b_rows * b_cols;
+    }
+    return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
+                       accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
 }

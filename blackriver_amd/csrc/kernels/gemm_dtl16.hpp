@@ -1,0 +1,355 @@
+// 16-bit MFMA GEMM, direct-to-LDS variant: the fast path for products whose
+// two operands are both stored in the MFMA element type (fp16 or bf16).
+//
+//   C[b][i,j] = alpha * sum_p opA[b][i,p] * opB[b][p,j] (+ C) (+ bias[j])
+//
+// Operand tiles never pass through registers on their way in: every wave
+// issues global_load_lds_dwordx4 (gfx950: 16 bytes per lane, 1 KiB per
+// instruction, written to LDS at M0 + lane*16).  Because the LDS side of such
+// a load is fixed to lane order, padding rows is not possible; bank conflicts
+// are avoided by choosing WHICH 16-byte chunk of the tile each lane fetches
+// (an XOR swizzle), and un-swizzling in the fragment reads:
+//
+//   k contiguous in memory  -> LDS image [row][4 chunks of 8 k], 64 bytes per
+//       row; chunk c of row r sits in slot c ^ ((r >> 2) & 3).  A fragment is
+//       one ds_read_b128 per lane; any 16 consecutive rows of one chunk column
+//       cover all 64 banks exactly once.
+//   row contiguous in memory-> LDS image [k][ROWS/8 chunks of 8 rows]; chunk c
+//       of k-row k sits in slot c ^ (4 * (k & 3)).  Fragments are read with
+//       ds_read_b64_tr_b16 (two per fragment); the 4 k-rows x 64 bytes that 32
+//       lanes touch in one pass land in 16 different 16-byte bank groups.
+//
+// Pipeline.  STAGES tile buffers form a ring and are all filled up front.  A K
+// step (KT = 32 or 64 k-values) is KT/16 sub-steps with two fragment register
+// sets used alternately:
+//   sub-step s < last:  issue the LDS reads of sub-step s+1, run the MFMAs of
+//       sub-step s (whose fragments were read one sub-step ago);
+//   last sub-step of tile t:  wait until this wave's loads of tile t+1 have
+//       landed (s_waitcnt vmcnt(N), later tiles stay in flight); workgroup
+//       barrier -- now tile t+1 is complete in LDS and every wave has read all
+//       of tile t; issue the loads of tile t+STAGES into the buffer tile t
+//       occupied; issue the LDS reads of (t+1, first sub-step); run the MFMAs.
+// KT = 64 makes a k-contiguous operand row a full 128-byte cache line per
+// step (with 32, each line is fetched from L2 twice, half used each time).
+// One barrier per K step, no staging registers, LDS latency hidden behind 16+
+// MFMAs inside the wave, HBM / L2 latency behind STAGES-1 K steps.  The loads
+// and the vmcnt waits are inline assembly because the compiler would otherwise
+// wait for ALL outstanding direct-to-LDS loads before any LDS read.
+//
+// Requirements (checked by the host dispatcher; everything else takes the
+// register-staged kernel in gemm_mfma16.hpp): K % 32 == 0, 16-byte aligned
+// operand bases / leading dimensions / batch strides, and for row-contiguous
+// operands rows % 8 == 0.  Rows past the end of an operand are redirected to a
+// valid row; their products land in rows / columns of C that are never stored.
+#pragma once
+
+#include "gemm_mfma16.hpp"
+
+#include <stdlib.h>
+#include <string.h>
+
+namespace brk {
+namespace gemm16 {
+
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+
+// One wave-wide direct-to-LDS load: lane l copies the 16 bytes at
+// sbase + voff(l) to LDS byte lds_dst + 16*l.
+__device__ __forceinline__ void dtl_load(unsigned lds_dst, unsigned voff, const void* sbase) {
+    asm volatile(
+        "s_mov_b32 m0, %0\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %1, %2"
+        :
+        : "s"(lds_dst), "v"(voff), "s"(sbase)
+        : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmem() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// Operand tile of ROWS x KT elements (KT = 32 or 64 k-values per K step).
+template <int ROWS, int KT, int WAVES, bool KSTR>
+struct DtlTile {
+    static constexpr int kBytes = ROWS * KT * 2;
+    static constexpr int kInstr = kBytes / 1024;     // wave-wide loads per tile
+    static constexpr int kPerWave = kInstr / WAVES;  // ... issued by each wave
+    static_assert(kInstr % WAVES == 0, "tile loads do not divide among the waves");
+    static_assert(ROWS >= 128, "swizzle needs at least 16 chunks per k-row");
+    // k contiguous: a row is KT/8 chunks; kRowsPer256 rows span the 64 banks
+    static constexpr int kRowBytes = KT * 2;
+    static constexpr int kChunksPerRow = KT / 8;
+    static constexpr int kRowsPer256 = 256 / kRowBytes;
+    static constexpr int kRowsPerInstr = 64 / kChunksPerRow;
+    // row contiguous: a k-row is ROWS/8 chunks
+    static constexpr int kChunksPerK = ROWS / 8;
+    static constexpr int kKPerInstr = 64 / kChunksPerK;
+
+    // Byte offset (from the tile origin at K step 0) of the chunk this lane
+    // fetches in its q-th load of a tile; LDS slot = instruction*64 + lane.
+    static __device__ __forceinline__ unsigned source_offset(int q, int wave, int lane, long long ld, long long row0,
+                                                             long long rows) {
+        const int j = q * WAVES + wave;
+        if (!KSTR) {
+            const int r = j * kRowsPerInstr + lane / kChunksPerRow;
+            const int c = (lane % kChunksPerRow) ^ ((r / kRowsPer256) % kChunksPerRow);
+            long long row = row0 + r;
+            row = row < rows ? row : rows - 1;
+            return (unsigned)(((row - row0) * ld + c * 8) * 2);
+        } else {
+            const int kk = j * kKPerInstr + lane / kChunksPerK;
+            const int c = (lane % kChunksPerK) ^ (4 * (kk & 3));
+            long long row = row0 + c * 8;
+            row = row < rows ? row : row0;
+            return (unsigned)((kk * ld + (row - row0)) * 2);
+        }
+    }
+
+    // LDS byte offset (inside one tile image) this lane reads the fragment of
+    // 32-row block `row_base` and 16-k sub-step ks from; row-contiguous tiles
+    // read a second time 4 k-rows further on.
+    static __device__ __forceinline__ unsigned frag_offset(int row_base, int ks, int lane) {
+        if (!KSTR) {
+            const int r = row_base + (lane & 31);
+            const int c = ks * 2 + (lane >> 5);
+            return (unsigned)(r * kRowBytes + ((c ^ ((r / kRowsPer256) % kChunksPerRow)) * 16));
+        } else {
+            const int i = lane & 15, grp = lane >> 4;
+            const int kk = ks * 16 + (grp >> 1) * 8 + (i >> 2);
+            const int row16 = row_base + (grp & 1) * 16 + (i & 3) * 4;
+            const int c = (row16 >> 3) ^ (4 * (i >> 2));
+            return (unsigned)(kk * (ROWS * 2) + c * 16 + (row16 & 7) * 2);
+        }
+    }
+
+    static __device__ __forceinline__ u32x4 fragment(const lds_byte* tile, unsigned off) {
+        if (!KSTR) {
+            return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(tile + off);
+        } else {
+            typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + off + 4 * ROWS * 2));
+            const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+            return mk4(l2.x, l2.y, h2.x, h2.y);
+        }
+    }
+};
+
+template <int CT, int BM, int BN, int WM, int WN, int KT, int STAGES, bool A_KSTR, bool B_KSTR, typename TC>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(GemmArgs g) {
+    constexpr int WAVES = (BM / WM) * (BN / WN);
+    constexpr int FM = WM / 32, FN = WN / 32, KS = KT / 16;
+    using TA = DtlTile<BM, KT, WAVES, A_KSTR>;
+    using TB = DtlTile<BN, KT, WAVES, B_KSTR>;
+    constexpr int kStageBytes = TA::kBytes + TB::kBytes;
+    constexpr int kLoads = TA::kPerWave + TB::kPerWave;  // per wave and tile
+    static_assert(STAGES >= 2 && STAGES <= 4, "two to four tile buffers");
+    static_assert(KT == 32 || KT == 64, "K tile of 32 or 64");
+    static_assert(STAGES * kStageBytes <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[STAGES * kStageBytes];
+    const lds_byte* lds = (const lds_byte*)lds_raw;
+    const unsigned lds0 = (unsigned)(unsigned long long)lds;
+
+    long long batch;
+    int tm, tn;
+    tile_coords(g, batch, tm, tn);
+    const long long row0 = (long long)tm * BM, col0 = (long long)tn * BN;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / (BN / WN), wn = wave % (BN / WN);
+
+    // tile origins at K step 0 (wave-uniform, advanced once per step) and the
+    // per-lane chunk offsets (fixed for the whole K loop)
+    const unsigned char* a_src = reinterpret_cast<const unsigned char*>(g.a) +
+                                 2 * (batch * g.sa + (A_KSTR ? row0 : row0 * g.lda));
+    const unsigned char* b_src = reinterpret_cast<const unsigned char*>(g.b) +
+                                 2 * (batch * g.sb + (B_KSTR ? col0 : col0 * g.ldb));
+    const long long a_step = A_KSTR ? 2 * KT * g.lda : 2 * KT;
+    const long long b_step = B_KSTR ? 2 * KT * g.ldb : 2 * KT;
+    unsigned a_off[TA::kPerWave], b_off[TB::kPerWave];
+#pragma unroll
+    for (int q = 0; q < TA::kPerWave; q++) a_off[q] = TA::source_offset(q, wave, lane, g.lda, row0, g.m);
+#pragma unroll
+    for (int q = 0; q < TB::kPerWave; q++) b_off[q] = TB::source_offset(q, wave, lane, g.ldb, col0, g.n);
+
+    unsigned fa_off[FM][KS], fb_off[FN][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+        for (int i = 0; i < FM; i++) fa_off[i][ks] = TA::frag_offset(wm * WM + i * 32, ks, lane);
+#pragma unroll
+        for (int j = 0; j < FN; j++) fb_off[j][ks] = TA::kBytes + TB::frag_offset(wn * WN + j * 32, ks, lane);
+    }
+
+    const int nk = (int)(g.k / KT);
+    auto issue = [&](int tile) {
+        const unsigned dst = lds0 + (unsigned)(tile % STAGES) * kStageBytes + (unsigned)wave * 1024u;
+#pragma unroll
+        for (int q = 0; q < TA::kPerWave; q++) dtl_load(dst + q * WAVES * 1024, a_off[q], a_src);
+#pragma unroll
+        for (int q = 0; q < TB::kPerWave; q++) dtl_load(dst + TA::kBytes + q * WAVES * 1024, b_off[q], b_src);
+        a_src += a_step;
+        b_src += b_step;
+    };
+    auto read_frags = [&](u32x4 (&fa)[FM], u32x4 (&fb)[FN], int tile, int ks) {
+        const lds_byte* stage = lds + (tile % STAGES) * kStageBytes;
+#pragma unroll
+        for (int i = 0; i < FM; i++) fa[i] = TA::fragment(stage, fa_off[i][ks]);
+#pragma unroll
+        for (int j = 0; j < FN; j++) fb[j] = TB::fragment(stage, fb_off[j][ks]);
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+    auto multiply = [&](const u32x4 (&fa)[FM], const u32x4 (&fb)[FN]) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++) acc[i][j] = Cvt<CT>::mfma(fa[i], fb[j], acc[i][j]);
+    };
+
+    // Fill the ring, wait for tile 0 and read its first sub-step of fragments.
+#pragma unroll
+    for (int s = 0; s < STAGES; s++)
+        if (s < nk) issue(s);
+    if (nk > STAGES - 1) {
+        wait_vmem<(STAGES - 1) * kLoads>();
+    } else {
+        wait_vmem<0>();
+    }
+    __syncthreads();
+    // Two fragment sets: while the MFMAs of one sub-step run, the LDS reads of
+    // the next sub-step are in flight.
+    u32x4 fa0[FM], fb0[FN], fa1[FM], fb1[FN];
+    read_frags(fa0, fb0, 0, 0);
+
+    for (int t = 0; t < nk; t++) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            u32x4(&fa_now)[FM] = (ks & 1) ? fa1 : fa0;
+            u32x4(&fb_now)[FN] = (ks & 1) ? fb1 : fb0;
+            u32x4(&fa_next)[FM] = (ks & 1) ? fa0 : fa1;
+            u32x4(&fb_next)[FN] = (ks & 1) ? fb0 : fb1;
+            if (ks + 1 < KS) {
+                read_frags(fa_next, fb_next, t, ks + 1);
+            } else if (t + 1 < nk) {
+                // tile t+1 has to be in LDS; the tiles issued after it may stay in flight
+                const int after = nk - 2 - t;
+                if (after >= STAGES - 2) {
+                    wait_vmem<(STAGES - 2) * kLoads>();
+                } else if (STAGES > 3 && after == 1) {
+                    wait_vmem<kLoads>();
+                } else {
+                    wait_vmem<0>();
+                }
+                // every wave has now read all of tile t, so its buffer can be refilled
+                __syncthreads();
+                if (t + STAGES < nk) issue(t + STAGES);
+                read_frags(fa_next, fb_next, t + 1, 0);
+            }
+            multiply(fa_now, fb_now);
+        }
+    }
+
+    // acc[i][j][v] is C[row, col] with
+    //   row = wm*WM + i*32 + (v/4)*8 + (lane/32)*4 + v%4,  col = wn*WN + j*32 + lane%32
+    TC* c_base = static_cast<TC*>(g.c) + batch * g.sc;
+#pragma unroll
+    for (int j = 0; j < FN; j++) {
+        const long long col = col0 + wn * WN + j * 32 + (lane & 31);
+        if (col >= g.n) continue;
+        const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+        for (int i = 0; i < FM; i++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const long long row = row0 + wm * WM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                if (row < g.m) {
+                    TC* p = c_base + row * g.ldc + col;
+                    float o = g.alpha * acc[i][j][v] + bias;
+                    if (g.accumulate) o += c_load<TC>(p);
+                    c_store<TC>(p, o);
+                }
+            }
+        }
+    }
+}
+
+// ---- host-side dispatch -------------------------------------------------------
+template <int CT, int BM, int BN, int WM, int WN, int KT, int ST>
+int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
+    constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+    g.tiles_m = (int)((g.m + BM - 1) / BM);
+    g.tiles_n = (int)((g.n + BN - 1) / BN);
+    const long long blocks = (long long)g.tiles_m * g.tiles_n * batch;
+    if (blocks > 0x7fffffffLL) return BR_ERR_ATTR;
+    const unsigned grid = (unsigned)blocks;
+    using F16 = __half;
+    using BF16 = __hip_bfloat16;
+#define BR_DTL_CASE(AK, BK_)                                                                           \
+    if (p.a_kstr == AK && p.b_kstr == BK_) {                                                            \
+        if (p.c_dtype == BR_F32)                                                                        \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, float><<<grid, THREADS, 0, st>>>(g);   \
+        else if (CT == BR_GEMM_F16)                                                                     \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, F16><<<grid, THREADS, 0, st>>>(g);     \
+        else                                                                                            \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, BF16><<<grid, THREADS, 0, st>>>(g);    \
+    }
+    BR_DTL_CASE(false, false)
+    BR_DTL_CASE(false, true)
+    BR_DTL_CASE(true, false)
+    BR_DTL_CASE(true, true)
+#undef BR_DTL_CASE
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+// The direct-to-LDS kernel applies when both operands are 16-bit, the fast
+// path's alignment rules hold and every per-lane source offset fits 32 bits.
+inline bool dtl_applies(const GemmArgs& g, const Problem& p) {
+    if (p.a_f32 || p.b_f32 || p.guarded) return false;
+    const long long lim = 1LL << 31;
+    const long long a_span = p.a_kstr ? 2 * 64 * g.lda : 2 * 256 * g.lda;
+    const long long b_span = p.b_kstr ? 2 * 64 * g.ldb : 2 * 256 * g.ldb;
+    return a_span < lim && b_span < lim;
+}
+
+// Tile choice: estimated time = rounds of workgroups over the 256 CUs x tile
+// area / relative MFMA rate of the configuration (measured on the BLOOM-7B1
+// linear-layer shapes: 256x256 ~ 1.0, 256x128 ~ 0.9, 128x128 ~ 0.8 with two
+// workgroups resident per CU).
+template <int CT>
+int launch_dtl(const GemmArgs& g, const Problem& p, long long batch, hipStream_t st) {
+    if (g.k % 64 != 0) return launch_dtl_config<CT, 128, 128, 64, 64, 32, 3>(g, p, batch, st);
+    auto rounds = [&](long long bm, long long bn, long long slots) {
+        const long long tiles = ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn) * batch;
+        return (double)((tiles + slots - 1) / slots);
+    };
+    const double c256 = rounds(256, 256, 256) * 256 * 256 / 1.0;
+    const double c256x128 = rounds(256, 128, 256) * 256 * 128 / 0.9;
+    const double c128 = rounds(128, 128, 512) * 2 * 128 * 128 / 0.8;
+    static const char* force = getenv("BR_GEMM_TILE");
+    int pick = c256 <= c256x128 && c256 <= c128 ? 0 : (c256x128 <= c128 ? 1 : 2);
+    if (force && strcmp(force, "256x256") == 0) pick = 0;
+    if (force && strcmp(force, "256x128") == 0) pick = 1;
+    if (force && strcmp(force, "128x128") == 0) pick = 2;
+    if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
+    if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
+    return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
+}
+
+template <int CT>
+int launch_any(const GemmArgs& g, const Problem& p, long long batch, hipStream_t st) {
+    if (dtl_applies(g, p)) return launch_dtl<CT>(g, p, batch, st);
+    return launch<CT>(g, p, batch, st);
+}
+
+}  // namespace gemm16
+}  // namespace brk

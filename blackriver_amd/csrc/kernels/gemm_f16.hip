@@ -1,8 +1,8 @@
 // fp16-multiplicand instantiations of the MFMA GEMM template.
-#include "gemm_mfma16.hpp"
+#include "gemm_dtl16.hpp"
 
 namespace brk {
 int gemm16_launch_f16(const gemm16::GemmArgs& g, const gemm16::Problem& p, long long batch, hipStream_t st) {
-    return gemm16::launch<BR_GEMM_F16>(g, p, batch, st);
+    return gemm16::launch_any<BR_GEMM_F16>(g, p, batch, st);
 }
 }  // namespace brk

@@ -399,7 +399,6 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_kernel(GemmAr
 struct Problem {
     bool a_f32, a_kstr, b_f32, b_kstr;
     int c_dtype;
-    bool big;      // 256x128 tiles instead of 128x128
     bool guarded;  // sizes / alignment rule out the fast kernel
 };
 
@@ -446,16 +445,14 @@ int launch_layout(const GemmArgs& g, const Problem& p, unsigned grid, hipStream_
     return BR_ERR_TODO;
 }
 
-// Fills in the tile counts for the chosen configuration and launches.
+// Fills in the tile counts and launches the register-staged kernel.
 template <int CT>
 int launch(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
-    const int bm = (p.big && !p.guarded) ? 256 : 128, bn = 128;
-    g.tiles_m = (int)((g.m + bm - 1) / bm);
-    g.tiles_n = (int)((g.n + bn - 1) / bn);
+    g.tiles_m = (int)((g.m + 127) / 128);
+    g.tiles_n = (int)((g.n + 127) / 128);
     const long long blocks = (long long)g.tiles_m * g.tiles_n * batch;
     if (blocks > 0x7fffffffLL) return BR_ERR_ATTR;
     if (p.guarded) return launch_layout<true, CT, 128, 128, 64, 64>(g, p, (unsigned)blocks, st);
-    if (p.big) return launch_layout<false, CT, 256, 128, 128, 64>(g, p, (unsigned)blocks, st);
     return launch_layout<false, CT, 128, 128, 64, 64>(g, p, (unsigned)blocks, st);
 }
 

@@ -209,6 +209,26 @@ int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float
                 int accumulate, void* c, int c_dtype, int64_t ldc, int64_t stride_c,
                 const float* bias, int64_t batch, int compute, br_stream_t stream);
 
+/* The same product for callers that can lend scratch memory.  fp32 operands
+ * are first converted to the 16-bit compute type into `workspace` (dense
+ * copies, one pass each), so that the product runs on the direct-to-LDS
+ * kernel that needs both operands in the MFMA type.  Replaces the same
+ * kernels::LtSgemm call (LtSgemm.cu:55-126); `workspace` plays the part of
+ * the scratch the reference hands to cublasLtMatmul (context.cpp:31).  Falls back to br_hip_gemm when `compute`
+ * is BR_GEMM_F32, no operand is fp32, the shape is not 16-byte friendly
+ * (k % 32, operand row lengths % 8) or the workspace is smaller than
+ * br_hip_gemm_staged_workspace() bytes.  Results are identical to
+ * br_hip_gemm's for the same `compute` (same rounding of the operands, same
+ * accumulation order within a tile configuration). */
+size_t br_hip_gemm_staged_workspace(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                                    int a_dtype, int b_dtype, int64_t batch);
+int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                       const void* a, int a_dtype, int64_t lda, int64_t stride_a,
+                       const void* b, int b_dtype, int64_t ldb, int64_t stride_b,
+                       int accumulate, void* c, int c_dtype, int64_t ldc, int64_t stride_c,
+                       const float* bias, int64_t batch, int compute,
+                       void* workspace, size_t workspace_bytes, br_stream_t stream);
+
 /* ---- data preparation (bit-exact integer / gather work) ---------------- */
 /* The embedding row gather of blackriver/train_bloom.cpp:50-56. */
 int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, int elem_bytes,
