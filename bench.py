@@ -10,10 +10,12 @@ product path: word script -> word machine -> TensorType -> HIPTensor -> HIP
 kernels.  Inputs and weights are resident in HBM before the timed region.
 
 One JSON line is printed.  Besides the step throughput it carries
-  roofline      the dominant kernel (the MFMA GEMM at the h->4h shape of this
-                block) timed on its own with HIP events on the launch stream
+  roofline      the dominant kernel (the direct-to-LDS MFMA GEMM at the h->4h
+                shape of this block) timed on its own with HIP events on the
+                launch stream
   elementwise   LayerNorm / bias-GELU / log-softmax+NLL kernels in GB/s
-  gemms         every GEMM shape of the block in TFLOP/s
+  gemms         every GEMM shape of the block in TFLOP/s, as the backend runs
+                it (fp32 operands staged to fp16) and the kernel alone
   cpu_baseline  the CPU oracle timed on the host cores on a bounded sample
 """
 from __future__ import annotations
@@ -114,28 +116,38 @@ def block_leg(args, host, hip, timer):
     return sec
 
 
-def gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch=1, iters=20):
+def gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch=1, iters=20, staged=False):
+    """Times one product.  staged=True goes through br_hip_gemm_staged the way
+    the tensor backend does (fp32 operands converted into a scratch block,
+    conversion time included)."""
     tt = {hip.F32: torch.float32, hip.F16: torch.float16}
     a = torch.randn((batch, m * k), device="cuda").to(tt[a_dt])
     b = torch.randn((batch, n * k), device="cuda").to(tt[b_dt])
     c = torch.empty((batch, m * n), device="cuda", dtype=tt[c_dt])
     lda, ldb = (m if ta else k), (k if tb else n)
     st = timer.stream
+    common = (ta, tb, m, n, k, 1.0, ctypes.c_void_p(a.data_ptr()), a_dt, lda, m * k, ctypes.c_void_p(b.data_ptr()),
+              b_dt, ldb, n * k, 0, ctypes.c_void_p(c.data_ptr()), c_dt, n, m * n, None, batch, hip.GEMM_F16)
+    if staged:
+        need = hip.load().br_hip_gemm_staged_workspace(ta, tb, m, n, k, a_dt, b_dt, batch)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
 
-    def fn(i):
-        hip.call("br_hip_gemm", ta, tb, m, n, k, 1.0, ctypes.c_void_p(a.data_ptr()), a_dt, lda, m * k,
-                 ctypes.c_void_p(b.data_ptr()), b_dt, ldb, n * k, 0, ctypes.c_void_p(c.data_ptr()), c_dt, n, m * n,
-                 None, batch, hip.GEMM_F16, st)
+        def fn(i):
+            hip.call("br_hip_gemm_staged", *common, ctypes.c_void_p(ws.data_ptr()), need, st)
+    else:
+        def fn(i):
+            hip.call("br_hip_gemm", *common, st)
     sec = timer.run(fn, iters, 3)
     return sec, 2.0 * m * n * k * batch
 
 
 def roofline_leg(hip, timer, torch, full):
-    """Dominant kernel: the fp16 MFMA GEMM, activations fp32 x weights fp16,
-    at the h->4h shape [2048 x 4096] . [16384 x 4096]^T of this block."""
+    """Dominant kernel: the direct-to-LDS fp16 MFMA GEMM at the h->4h shape
+    [2048 x 4096] . [16384 x 4096]^T of this block, operands as the tensor
+    backend hands them to it (activations already converted to fp16)."""
     f32, f16 = hip.F32, hip.F16
-    sec, flop = gemm_case(hip, timer, torch, 0, 1, N, F, H, f32, f16, f32, iters=30)
-    roof = {"bound": "mfma", "kernel": "gemm_mfma16_kernel (A fp32 row-major, B fp16 [n,k], C fp32)",
+    sec, flop = gemm_case(hip, timer, torch, 0, 1, N, F, H, f16, f16, f32, iters=30)
+    roof = {"bound": "mfma", "kernel": "gemm_dtl_kernel 256x256x64 (A fp16 [m,k], B fp16 [n,k], C fp32)",
             "shape": "m=%d n=%d k=%d" % (N, F, H), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, "us_per_launch": sec * 1e6,
             "traffic": None}
@@ -155,9 +167,13 @@ def roofline_leg(hip, timer, torch, full):
             ("dV=P^T.dO", 1, 0, T, hd, T, f32, f32, f32, B * NH),
         ]
         for name, ta, tb, m, n, k, a, b, c, batch in cases:
-            s, fl = gemm_case(hip, timer, torch, ta, tb, m, n, k, a, b, c, batch, iters=10)
+            # as the backend runs it (fp32 activations staged to fp16) and the kernel alone on fp16 operands
+            s, fl = gemm_case(hip, timer, torch, ta, tb, m, n, k, a, b, c, batch, iters=10, staged=True)
+            s16, _ = gemm_case(hip, timer, torch, ta, tb, m, n, k, f16, f16, c, batch, iters=10)
             gemms.append({"name": name, "m": m, "n": n, "k": k, "batch": batch, "us": round(s * 1e6, 1),
-                          "tflops": round(fl / s / 1e12, 1), "frac": round(fl / s / 1e12 / MFMA_F16_PEAK_TFLOPS, 3)})
+                          "tflops": round(fl / s / 1e12, 1), "kernel_us": round(s16 * 1e6, 1),
+                          "kernel_tflops": round(fl / s16 / 1e12, 1),
+                          "kernel_frac": round(fl / s16 / 1e12 / MFMA_F16_PEAK_TFLOPS, 3)})
     return roof, gemms
 
 
