@@ -343,6 +343,98 @@ __global__ __launch_bounds__(kBlock) void colsum_final(const float* partial, flo
     out[col] = acc;
 }
 
+// Vector forms of the two stages (cols % VEC == 0, 16-byte aligned rows).
+// Stage 1: a thread owns VEC adjacent columns and sums a strip of rows, four
+// rows of loads in flight at a time.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kBlock) void colsum_partial_vec(const T* __restrict__ x, float* __restrict__ partial,
+                                                              int64_t rows, int64_t cols, int rows_per_block) {
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (col >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[j] = 0.f;
+    int64_t r = r0;
+    for (; r + 4 <= r1; r += 4) {
+        float v[4][VEC];
+#pragma unroll
+        for (int u = 0; u < 4; u++) VecIO<T, VEC>::load(x + (r + u) * cols + col, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[j] += v[u][j];
+    }
+    for (; r < r1; r++) {
+        float v[VEC];
+        VecIO<T, VEC>::load(x + r * cols + col, v);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) acc[j] += v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) partial[(int64_t)blockIdx.y * cols + col + j] = acc[j];
+}
+
+// Stage 2 for cols % 4 == 0: 1024 threads = 16 column quads x 64 slices of
+// groups, every load of a workgroup in flight at once; slices are combined in
+// LDS in a fixed order.
+__global__ __launch_bounds__(1024) void colsum_final_x4(const float4* __restrict__ partial, float4* __restrict__ out,
+                                                        int groups, int cols4) {
+    __shared__ float4 l[64][16];
+    const int q = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int c4 = blockIdx.x * 16 + q;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c4 < cols4) {
+#pragma unroll 4
+        for (int g = sl; g < groups; g += 64) {
+            const float4 a = partial[(int64_t)g * cols4 + c4];
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        }
+    }
+    l[sl][q] = s;
+    __syncthreads();
+    if (sl < 8) {
+        for (int k = sl + 8; k < 64; k += 8) {
+            const float4 a = l[k][q];
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        }
+        l[sl][q] = s;
+    }
+    __syncthreads();
+    if (sl == 0 && c4 < cols4) {
+        for (int k = 1; k < 8; k++) {
+            const float4 a = l[k][q];
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
+        }
+        out[c4] = s;
+    }
+}
+
+// Launches stage 2 in its vector form when the shapes allow.
+int colsum_finish(const float* partial, float* out, int groups, int64_t cols, hipStream_t st) {
+    if (cols % 4 == 0 && aligned16(partial) && aligned16(out))
+        colsum_final_x4<<<(unsigned)((cols / 4 + 15) / 16), 1024, 0, st>>>(reinterpret_cast<const float4*>(partial),
+                                                                            reinterpret_cast<float4*>(out), groups,
+                                                                            (int)(cols / 4));
+    else
+        colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>(partial, out, groups, cols);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+// Row strips of the vector column sum: about 1024 workgroups in all, at most
+// 256 strips.
+constexpr int kMaxColsumGroups = 256;
+int colsum_vec_rows_per_block(int64_t rows, int64_t blocks_x) {
+    int64_t groups = 1024 / (blocks_x < 1 ? 1 : blocks_x);
+    if (groups < 1) groups = 1;
+    if (groups > kMaxColsumGroups) groups = kMaxColsumGroups;
+    int64_t rpb = (rows + groups - 1) / groups;
+    if (rpb < 4) rpb = 4;
+    return (int)rpb;
+}
+
 // ------------------------------------------------------- transpose 0213
 // One 16-byte granule per thread, indexed by OUTPUT position so stores are
 // fully coalesced; loads are contiguous runs of s3 elements.
@@ -623,12 +715,7 @@ int br_hip_gelu_bwd(const void* dy, const void* x, void* dx, int dtype, int64_t 
     return BR_OK;
 }
 
-size_t br_hip_bias_gelu_bwd_workspace(int64_t rows, int64_t cols) {
-    if (rows <= 0 || cols <= 0) return 0;
-    const int rpb = strip_rows(rows);
-    const int64_t groups = (rows + rpb - 1) / rpb;
-    return (size_t)(groups * cols) * sizeof(float);
-}
+size_t br_hip_bias_gelu_bwd_workspace(int64_t rows, int64_t cols) { return br_hip_colsum_workspace(rows, cols); }
 
 int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void* dx, float* dbias, int dtype,
                          int64_t rows, int64_t cols, void* workspace, size_t workspace_bytes,
@@ -669,15 +756,16 @@ int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void*
         return BR_OK;
     }
     BR_HIP_LAUNCH_CHECK();
-    if (dbias) {
-        colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>(partial, dbias, groups, cols);
-        BR_HIP_LAUNCH_CHECK();
-    }
+    if (dbias) return colsum_finish(partial, dbias, groups, cols, st);
     return BR_OK;
 }
 
 size_t br_hip_colsum_workspace(int64_t rows, int64_t cols) {
-    return br_hip_bias_gelu_bwd_workspace(rows, cols);
+    if (rows <= 0 || cols <= 0) return 0;
+    const int rpb = strip_rows(rows);
+    const size_t strips = (size_t)((rows + rpb - 1) / rpb) * (size_t)cols * sizeof(float);
+    const size_t vec = (size_t)kMaxColsumGroups * (size_t)cols * sizeof(float);
+    return strips > vec ? strips : vec;
 }
 
 int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols, void* workspace,
@@ -688,20 +776,30 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
     if (rows == 0) return br_hip_fill(out, BR_F32, 0.f, cols, stream);
     if (!x) return BR_ERR_INPUT;
     if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
+    if (dtype != BR_F32 && dtype != BR_F16) return BR_ERR_TODO;
+    float* partial = (float*)workspace;
+    const int vec = dtype == BR_F32 ? 4 : 8;
+    if (cols % vec == 0 && aligned16(x) && (cols * (dtype == BR_F32 ? 4 : 2)) % 16 == 0) {
+        const int64_t blocks_x = (cols / vec + kBlock - 1) / kBlock;
+        const int rpb = colsum_vec_rows_per_block(rows, blocks_x);
+        const int groups = (int)((rows + rpb - 1) / rpb);
+        dim3 grid((unsigned)blocks_x, (unsigned)groups);
+        if (dtype == BR_F32)
+            colsum_partial_vec<float, 4><<<grid, kBlock, 0, st>>>((const float*)x, partial, rows, cols, rpb);
+        else
+            colsum_partial_vec<__half, 8><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
+        BR_HIP_LAUNCH_CHECK();
+        return colsum_finish(partial, out, groups, cols, st);
+    }
     const int rpb = strip_rows(rows);
     const int groups = (int)((rows + rpb - 1) / rpb);
     dim3 grid((unsigned)((cols + kBlock - 1) / kBlock), (unsigned)groups);
     if (dtype == BR_F32)
-        colsum_partial<float><<<grid, kBlock, 0, st>>>((const float*)x, (float*)workspace, rows, cols, rpb);
-    else if (dtype == BR_F16)
-        colsum_partial<__half><<<grid, kBlock, 0, st>>>((const __half*)x, (float*)workspace, rows, cols, rpb);
+        colsum_partial<float><<<grid, kBlock, 0, st>>>((const float*)x, partial, rows, cols, rpb);
     else
-        return BR_ERR_TODO;
+        colsum_partial<__half><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
-    colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>((const float*)workspace, out,
-                                                                               groups, cols);
-    BR_HIP_LAUNCH_CHECK();
-    return BR_OK;
+    return colsum_finish(partial, out, groups, cols, st);
 }
 
 int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, int64_t s1, int64_t s2,

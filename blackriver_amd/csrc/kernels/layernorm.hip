@@ -11,6 +11,8 @@
 // workspace and a small second kernel adds them in a fixed order.
 #include "common.hpp"
 
+#include <stdlib.h>
+
 using namespace brk;
 
 namespace {
@@ -128,18 +130,25 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* __restrict__ 
         acc_g[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         acc_b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    int flip = 0;
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, flip ^= 1) {
+    // The next row's dy / y are requested before the current row is worked on,
+    // so two rows per workgroup are in flight.
+    float4 d[VPT], xh[VPT], nd[VPT], nxh[VPT];
+    auto request = [&](float4 (&rd)[VPT], float4 (&ry)[VPT], int64_t row) {
         const float4* dyr = reinterpret_cast<const float4*>(dy) + row * cols4;
         const float4* yr = reinterpret_cast<const float4*>(y) + row * cols4;
-        float4 d[VPT], xh[VPT];
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
             const int idx = threadIdx.x + i * kBlock;
             const bool ok = idx < cols4;
-            d[i] = ok ? dyr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-            xh[i] = ok ? yr[idx] : b[i];
+            rd[i] = ok ? dyr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+            ry[i] = ok ? yr[idx] : b[i];
         }
+    };
+    if (blockIdx.x < rows) request(d, xh, blockIdx.x);
+    int flip = 0;
+    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, flip ^= 1) {
+        const int64_t next = row + gridDim.x;
+        if (next < rows) request(nd, nxh, next);
         // stored var already holds eps; the backward adds eps once more
         const float rstd = 1.0f / sqrtf(var[row] + eps);
         float s[2] = {0.f, 0.f};
@@ -171,6 +180,11 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* __restrict__ 
                 o.w = (d[i].w - m1 - xh[i].w * m2) * rstd;
                 dxr[idx] = o;
             }
+        }
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            d[i] = nd[i];
+            xh[i] = nxh[i];
         }
     }
     float4* pg = reinterpret_cast<float4*>(part_dgamma) + (int64_t)blockIdx.x * cols4;
@@ -251,9 +265,55 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_finalize(const float* part_dgam
     }
 }
 
+// The same sums for the register path's partials (cols % 4 == 0, 16-byte
+// aligned): 1024 threads = 16 column quads x 64 slices of partials, so that
+// all of a workgroup's loads are in flight at once; slices are combined in LDS
+// in a fixed order.
+constexpr int kFinSlices = 64;
+__global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restrict__ part_dgamma,
+                                                           const float4* __restrict__ part_dbeta,
+                                                           float4* __restrict__ dgamma, float4* __restrict__ dbeta,
+                                                           int parts, int cols4) {
+    __shared__ float4 lg[kFinSlices][16], lb[kFinSlices][16];
+    const int q = threadIdx.x & 15, sl = threadIdx.x >> 4;
+    const int c4 = blockIdx.x * 16 + q;
+    float4 sg = make_float4(0.f, 0.f, 0.f, 0.f), sb = sg;
+    if (c4 < cols4) {
+#pragma unroll 8
+        for (int p = sl; p < parts; p += kFinSlices) {
+            const float4 a = part_dgamma[(int64_t)p * cols4 + c4], b = part_dbeta[(int64_t)p * cols4 + c4];
+            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
+            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+        }
+    }
+    lg[sl][q] = sg;
+    lb[sl][q] = sb;
+    __syncthreads();
+    if (sl < 8) {
+        for (int k = sl + 8; k < kFinSlices; k += 8) {
+            const float4 a = lg[k][q], b = lb[k][q];
+            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
+            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+        }
+        lg[sl][q] = sg;
+        lb[sl][q] = sb;
+    }
+    __syncthreads();
+    if (sl == 0 && c4 < cols4) {
+        for (int k = 1; k < 8; k++) {
+            const float4 a = lg[k][q], b = lb[k][q];
+            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
+            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+        }
+        dgamma[c4] = sg;
+        dbeta[c4] = sb;
+    }
+}
+
 int bwd_parts(int64_t rows) {
     // persistent workgroups: two per CU on a 256-CU part, never more than rows
-    int64_t p = 512;
+    static const char* e = getenv("BR_LN_PARTS");
+    int64_t p = e ? atoi(e) : 512;
     if (p > rows) p = rows;
     return (int)(p < 1 ? 1 : p);
 }
@@ -338,7 +398,12 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, co
         else
             ln_bwd_regs<8><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
         BR_HIP_LAUNCH_CHECK();
-        ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols);
+        if (aligned16(dgamma) && aligned16(dbeta))
+            ln_bwd_finalize_x4<<<(unsigned)((cols4 + 15) / 16), 1024, 0, st>>>(
+                reinterpret_cast<const float4*>(part_g), reinterpret_cast<const float4*>(part_b),
+                reinterpret_cast<float4*>(dgamma), reinterpret_cast<float4*>(dbeta), parts, cols4);
+        else
+            ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols);
     } else {
         const int rpb = strip_rows(rows);
         parts = (int)((rows + rpb - 1) / rpb);
