@@ -71,9 +71,24 @@ int product(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alp
         return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
                            accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
     const size_t need = br_hip_gemm_staged_workspace(trans_a, trans_b, m, n, k, a_dtype, b_dtype, batch);
-    void* ws = ComputingContext::gemm_staging(need);
+    void* ws = ComputingContext::gemm_staging(0, need);
     return br_hip_gemm_staged(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
                               accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, ws, need, stream);
+}
+
+// An operand that several products of one operator read: with a 16-bit MFMA
+// type an fp32 operand is converted once here (same rounding as the staged
+// GEMM entry point applies), otherwise it is passed through.
+struct Operand {
+    const void* ptr;
+    int dtype;
+};
+Operand shared_operand(const void* p, int dtype, int64_t items, int compute) {
+    if (dtype != BR_F32 || compute == BR_GEMM_F32 || items % 8 != 0) return {p, dtype};
+    const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
+    void* dst = ComputingContext::gemm_staging(1, (size_t)items * 2);
+    BR_HIP_CHECK(br_hip_cast(p, BR_F32, dst, native, items, ComputingContext::stream));
+    return {dst, native};
 }
 
 // fp32 device pointer to a bias vector, converting 16-bit storage on the fly
@@ -519,11 +534,12 @@ ComputingReturn HIPTensor<DT>::op_linear_backward(tensor_t self, tensor_t x, ten
     void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
     BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, ws, need, stream()));
     // weight_g[out,in] = dy^T . x
-    BR_OP(product(1, 0, out, in, n, 1.0f, mem_, (int)DT, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
-                      code(weight_g), in, 0, nullptr, 1, compute));
+    const Operand dy = shared_operand(mem_, (int)DT, n * out, compute);
+    BR_OP(product(1, 0, out, in, n, 1.0f, dy.ptr, dy.dtype, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
+                  code(weight_g), in, 0, nullptr, 1, compute));
     // x_g[n,in] = dy . W
-    BR_OP(product(0, 0, n, in, out, 1.0f, mem_, (int)DT, out, 0, weight->data(), code(weight), in, 0, 0,
-                      x_g->data(), code(x_g), in, 0, nullptr, 1, compute));
+    BR_OP(product(0, 0, n, in, out, 1.0f, dy.ptr, dy.dtype, out, 0, weight->data(), code(weight), in, 0, 0,
+                  x_g->data(), code(x_g), in, 0, nullptr, 1, compute));
     return OP_OK;
 }
 
@@ -588,11 +604,12 @@ ComputingReturn HIPTensor<DT>::op_softmax_attn_backward(tensor_t self, tensor_t 
     if (!dev_f32(attn_g) || !dev(v_g) || attn_g->items() != attn->items() || v_g->items() != v->items())
         return OP_OUTPUT_ERROR;
     const int compute = pick_compute({self, attn, v});
-    BR_OP(product(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, mem_, (int)DT, d.hd,
-                      d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute));
+    const Operand d_o = shared_operand(mem_, (int)DT, d.bh * d.t * d.hd, compute);
+    BR_OP(product(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, d_o.ptr, d_o.dtype, d.hd,
+                  d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute));
     float* dp = static_cast<float*>(ComputingContext::scratch((size_t)(d.bh * d.t * d.t) * sizeof(float)));
-    BR_OP(product(0, 1, d.t, d.t, d.hd, 1.0f, mem_, (int)DT, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
-                      d.t * d.hd, 0, dp, BR_F32, d.t, d.t * d.t, nullptr, d.bh, compute));
+    BR_OP(product(0, 1, d.t, d.t, d.hd, 1.0f, d_o.ptr, d_o.dtype, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
+                  d.t * d.hd, 0, dp, BR_F32, d.t, d.t * d.t, nullptr, d.bh, compute));
     BR_OP(br_hip_softmax_bwd(dp, static_cast<const float*>(attn->data()), static_cast<float*>(attn_g->data()),
                              d.bh * d.t, d.t, stream()));
     return OP_OK;
@@ -608,10 +625,11 @@ ComputingReturn HIPTensor<DT>::op_qk_backward(tensor_t self, tensor_t q, tensor_
     if (!dev(q_g) || !dev(k_g) || q_g->items() != q->items() || k_g->items() != q->items()) return OP_OUTPUT_ERROR;
     const float alpha = (float)(1.0 / sqrt((double)hd));
     const int compute = pick_compute({self, q, k});
-    BR_OP(product(0, 0, t, hd, t, alpha, mem_, (int)DT, t, t * t, k->data(), code(k), hd, t * hd, 0, q_g->data(),
-                      code(q_g), hd, t * hd, nullptr, bh, compute));
-    BR_OP(product(1, 0, t, hd, t, alpha, mem_, (int)DT, t, t * t, q->data(), code(q), hd, t * hd, 0, k_g->data(),
-                      code(k_g), hd, t * hd, nullptr, bh, compute));
+    const Operand ds = shared_operand(mem_, (int)DT, bh * t * t, compute);
+    BR_OP(product(0, 0, t, hd, t, alpha, ds.ptr, ds.dtype, t, t * t, k->data(), code(k), hd, t * hd, 0, q_g->data(),
+                  code(q_g), hd, t * hd, nullptr, bh, compute));
+    BR_OP(product(1, 0, t, hd, t, alpha, ds.ptr, ds.dtype, t, t * t, q->data(), code(q), hd, t * hd, 0, k_g->data(),
+                  code(k_g), hd, t * hd, nullptr, bh, compute));
     return OP_OK;
 }
 

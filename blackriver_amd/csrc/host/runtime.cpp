@@ -54,8 +54,8 @@ size_t ComputingContext::workspace_size = 0;
 int ComputingContext::fp32_gemm_compute = BR_GEMM_F32;
 void* ComputingContext::scratch_ptr_ = nullptr;
 size_t ComputingContext::scratch_size_ = 0;
-void* ComputingContext::staging_ptr_ = nullptr;
-size_t ComputingContext::staging_size_ = 0;
+void* ComputingContext::staging_ptr_[2] = {nullptr, nullptr};
+size_t ComputingContext::staging_size_[2] = {0, 0};
 
 void ComputingContext::boot(int dev) {
     br_assert(device < 0, "ComputingContext is already booted");
@@ -73,11 +73,15 @@ void ComputingContext::shutdown() {
     sync();
     free(host_workspace);
     if (scratch_ptr_) BR_HIP_CHECK(br_hip_free(scratch_ptr_));
-    if (staging_ptr_) BR_HIP_CHECK(br_hip_free(staging_ptr_));
+    for (int i = 0; i < 2; i++) {
+        if (staging_ptr_[i]) BR_HIP_CHECK(br_hip_free(staging_ptr_[i]));
+        staging_ptr_[i] = nullptr;
+        staging_size_[i] = 0;
+    }
     BR_HIP_CHECK(br_hip_free(workspace));
     BR_HIP_CHECK(br_hip_stream_destroy(stream));
-    host_workspace = workspace = stream = scratch_ptr_ = staging_ptr_ = nullptr;
-    workspace_size = scratch_size_ = staging_size_ = 0;
+    host_workspace = workspace = stream = scratch_ptr_ = nullptr;
+    workspace_size = scratch_size_ = 0;
     device = -1;
 }
 
@@ -99,17 +103,19 @@ void* ComputingContext::scratch(size_t bytes) {
     return scratch_ptr_;
 }
 
-void* ComputingContext::gemm_staging(size_t bytes) {
+void* ComputingContext::gemm_staging(int slot, size_t bytes) {
     br_assert(device >= 0, "ComputingContext is not booted");
-    if (bytes > staging_size_) {
+    br_assert(slot == 0 || slot == 1, "staging slot");
+    if (bytes > staging_size_[slot]) {
+        // earlier kernels on the stream may still be using the old block
         sync();
-        if (staging_ptr_) BR_HIP_CHECK(br_hip_free(staging_ptr_));
+        if (staging_ptr_[slot]) BR_HIP_CHECK(br_hip_free(staging_ptr_[slot]));
         // room to spare, so that a slightly larger product does not reallocate
         bytes += bytes / 4;
-        BR_HIP_CHECK(br_hip_malloc(&staging_ptr_, bytes));
-        staging_size_ = bytes;
+        BR_HIP_CHECK(br_hip_malloc(&staging_ptr_[slot], bytes));
+        staging_size_[slot] = bytes;
     }
-    return staging_ptr_;
+    return staging_ptr_[slot];
 }
 
 // ----------------------------------------------------- CollectiveContext

@@ -33,15 +33,17 @@ struct ComputingContext {
     // Grow-only device scratch for operators whose need exceeds `workspace`
     // (the attention backward stages dP for all heads at once).
     static void* scratch(size_t bytes);
-    // Grow-only device block of its own for the 16-bit operand copies the
-    // GEMM entry point stages (never the workspace: operands may live there).
-    static void* gemm_staging(size_t bytes);
+    // Grow-only device blocks of their own for 16-bit copies of fp32 GEMM
+    // operands (never the workspace: operands may live there).  Slot 0 is what
+    // the staged GEMM entry point converts into, slot 1 holds an operand that
+    // several products of one operator share.
+    static void* gemm_staging(int slot, size_t bytes);
 
 private:
     static void* scratch_ptr_;
     static size_t scratch_size_;
-    static void* staging_ptr_;
-    static size_t staging_size_;
+    static void* staging_ptr_[2];
+    static size_t staging_size_[2];
 };
 
 // One process, one GPU: rank 0 of a world of 1.  `now()` keeps feeding the

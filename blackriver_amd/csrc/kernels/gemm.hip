@@ -289,8 +289,38 @@ __global__ __launch_bounds__(256) void stage_rows_kernel(const float* __restrict
     }
 }
 
+// Dense operand (rows follow each other without gaps): a flat conversion, 8
+// elements per thread, no index arithmetic.
+template <bool BF>
+__global__ __launch_bounds__(256) void stage_flat_kernel(const float4* __restrict__ src, gemm16::u32x4* __restrict__ dst,
+                                                         long long n8) {
+    for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < n8;
+         i += (long long)gridDim.x * blockDim.x) {
+        const float4 a = src[2 * i], b = src[2 * i + 1];
+        constexpr int CT = BF ? BR_GEMM_BF16 : BR_GEMM_F16;
+        gemm16::u32x4 o;
+        o.x = gemm16::pack2(gemm16::Cvt<CT>::from_f32(a.x), gemm16::Cvt<CT>::from_f32(a.y));
+        o.y = gemm16::pack2(gemm16::Cvt<CT>::from_f32(a.z), gemm16::Cvt<CT>::from_f32(a.w));
+        o.z = gemm16::pack2(gemm16::Cvt<CT>::from_f32(b.x), gemm16::Cvt<CT>::from_f32(b.y));
+        o.w = gemm16::pack2(gemm16::Cvt<CT>::from_f32(b.z), gemm16::Cvt<CT>::from_f32(b.w));
+        dst[i] = o;
+    }
+}
+
 int stage_rows(const float* src, long long ld, long long stride, long long rows, long long cols, long long batch,
                void* dst, int compute, hipStream_t st) {
+    const long long total = batch * rows * cols;
+    if (ld == cols && (batch == 1 || stride == rows * cols) && total % 8 == 0 && aligned16(src) && aligned16(dst)) {
+        const unsigned grid = grid_for(total / 8, 256, 1 << 14);
+        if (compute == BR_GEMM_F16)
+            stage_flat_kernel<false><<<grid, 256, 0, st>>>(reinterpret_cast<const float4*>(src),
+                                                           static_cast<gemm16::u32x4*>(dst), total / 8);
+        else
+            stage_flat_kernel<true><<<grid, 256, 0, st>>>(reinterpret_cast<const float4*>(src),
+                                                          static_cast<gemm16::u32x4*>(dst), total / 8);
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
+    }
     const bool vec = cols % 4 == 0 && ld % 4 == 0 && stride % 4 == 0 && aligned16(src) && aligned16(dst);
     const long long work = batch * rows * (vec ? cols / 4 : cols);
     const unsigned grid = grid_for(work, 256, 1 << 16);
