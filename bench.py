@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BLOOM-7B1 training hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--leg all|block|roofline|elementwise]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--leg all|block|roofline|elementwise|copy]
 
 A "step" is one forward + backward pass of one BLOOM-7B1 decoder block
 (hidden 4096, 32 heads x 128, FFN 16384, ALiBi causal attention, batch 4 x
@@ -34,6 +34,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16
+# HBM bytes per launch of the roofline kernel at the roofline shape, from the
+# FETCH_SIZE / WRITE_SIZE counters of rocprofv3, each scaled by what the same
+# counter reads on the copy leg (402.5 MB fetched + 134.2 MB written).
+ROOFLINE_TRAFFIC_BYTES = 536.7e6
 
 H, NH, F, V = 4096, 32, 16384, 250880
 B, T = 4, 512
@@ -48,7 +52,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--leg", default="all", choices=["all", "block", "roofline", "elementwise"])
+    ap.add_argument("--leg", default="all", choices=["all", "block", "roofline", "elementwise", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     return ap.parse_args()
 
@@ -150,7 +154,7 @@ def roofline_leg(hip, timer, torch, full):
     roof = {"bound": "mfma", "kernel": "gemm_dtl_kernel 256x256x64 (A fp16 [m,k], B fp16 [n,k], C fp32)",
             "shape": "m=%d n=%d k=%d" % (N, F, H), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, "us_per_launch": sec * 1e6,
-            "traffic": None}
+            "traffic": ROOFLINE_TRAFFIC_BYTES}
     gemms = []
     if full:
         hd = H // NH
@@ -240,6 +244,22 @@ def elementwise_leg(hip, timer, torch):
     return out
 
 
+def copy_leg(hip, timer, torch):
+    """A plain copy kernel of known size (256 MiB read, 256 MiB written per
+    launch): the yardstick the FETCH_SIZE / WRITE_SIZE counters of the GEMM are
+    scaled by."""
+    n = 64 << 20
+    src = torch.randn(n, device="cuda")
+    dst = torch.empty(n, device="cuda")
+    st = timer.stream
+
+    def fn(i):
+        hip.call("br_hip_cast", ctypes.c_void_p(src.data_ptr()), hip.F32, ctypes.c_void_p(dst.data_ptr()), hip.F32, n, st)
+    sec = timer.run(fn, 10, 2)
+    return {"kernel": "cast_x8_kernel<float, float>", "bytes_read": 4 * n, "bytes_written": 4 * n,
+            "us": sec * 1e6, "GB/s": 8 * n / sec / 1e9}
+
+
 def cpu_baseline_leg():
     """The CPU oracle (a restatement of the reference's operators; the
     reference itself has no CPU math path) on a bounded sample: the same
@@ -300,6 +320,8 @@ def main():
             result["gemms"] = gemms
     if args.leg in ("all", "elementwise"):
         result["elementwise"] = elementwise_leg(hip, timer, torch)
+    if args.leg == "copy":
+        result["copy"] = copy_leg(hip, timer, torch)
     if args.leg == "all" and not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline_leg()
     host.sync()
