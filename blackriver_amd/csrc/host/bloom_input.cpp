@@ -90,9 +90,31 @@ struct XMask : public NativeWord {
     NWORD_CREATOR_DEFINE_LR(XMask)
 };
 
+// ( tensor mean std seed -- )  synthetic initialisation of a device tensor
+struct Normal : public NativeWord {
+    void run(Stack& stack) override {
+        const double seed = stack.pop_number();
+        const double std = stack.pop_number();
+        const double mean = stack.pop_number();
+        tensor_t t = stack.pop_tensor();
+        br_assert(t->is_cuda() && t->dtype() != DataType::Int, "bloom.normal: expects a device float tensor");
+        BR_HIP_CHECK(br_hip_normal(t->data(), (int)t->dtype(), (float)mean, (float)std, (uint64_t)seed,
+                                   (int64_t)t->items(), ComputingContext::stream));
+    }
+    NWORD_CREATOR_DEFINE_LR(Normal)
+};
+
+// ( -- loss )  what the most recent op.loss_backward returned
+struct LastLoss : public NativeWord {
+    void run(Stack& stack) override { stack.push_number((double)ComputingContext::last_loss); }
+    NWORD_CREATOR_DEFINE_LR(LastLoss)
+};
+
 }  // namespace
 
 void load_bloom_words(Enviroment& env) {
+    env.insert_native_word("bloom.normal", Normal::creator);
+    env.insert_native_word("bloom.last_loss", LastLoss::creator);
     env.insert_native_word("bloom.embed", Embed::creator);
     env.insert_native_word("bloom.alibi", Alibi::creator);
     env.insert_native_word("bloom.xmask", XMask::creator);

@@ -1,0 +1,117 @@
+#include "bloom_trainer.hpp"
+
+#include <cstring>
+#include <sstream>
+
+#include "common.hpp"
+#include "runtime.hpp"
+#include "tensor.hpp"
+
+namespace br {
+
+BloomTrainer::BloomTrainer(Enviroment& env, const BloomModelConfig& cfg) : env_(env), cfg_(cfg) {
+    br_assert(cfg.layers >= 1, "a model needs at least one block");
+    br_assert(cfg.hidden % cfg.heads == 0, "hidden size must divide among the heads");
+    br_assert(cfg.batch >= 1 && cfg.tokens >= 2, "batch >= 1 and tokens >= 2");
+    br_assert((size_t)cfg.layers + 1 <= env.hashes_num(), "the environment has too few hashes for the layers");
+}
+
+// The carve-up of create_dynamic_here (bloom.words): ten [B,T,H] buffers, two
+// [B,T,4H], alibi, three [H] statistics vectors, xmask and the probabilities.
+int64_t BloomTrainer::block_arena_floats() const {
+    const int64_t bth = cfg_.batch * cfg_.tokens * cfg_.hidden;
+    return 10 * bth + 2 * 4 * bth + cfg_.heads * cfg_.tokens + 3 * cfg_.hidden +
+           cfg_.batch * cfg_.tokens * cfg_.tokens + cfg_.batch * cfg_.heads * cfg_.tokens * cfg_.tokens;
+}
+
+int64_t BloomTrainer::model_arena_floats() const {
+    // plus one logits row per position: the loss head then needs a single group
+    return block_arena_floats() + cfg_.batch * cfg_.tokens * cfg_.vocab;
+}
+
+std::string BloomTrainer::setup_script() const {
+    std::ostringstream s;
+    s.precision(9);
+    auto dims = [&]() {
+        s << cfg_.hidden << " " << cfg_.heads << " " << cfg_.vocab << " " << cfg_.eps << " model_dims\n";
+        s << "'cuda' $DEVICE !  '" << cfg_.weight_dtype << "' $WDTYPE !\n";
+    };
+    s << "0 #\n";
+    dims();
+    s << "'" << cfg_.gemm_precision << "' op.gemm_precision\n";
+    s << "create_model_weight create_model_grad\n";
+    s << model_arena_floats() << " create_var\n";
+    s << cfg_.batch << " " << cfg_.tokens << " create_model_dynamic\n";
+    for (int i = 1; i <= cfg_.layers; i++) {
+        s << i << " #\n";
+        dims();
+        s << "create_layer_weight create_layer_grad\n";
+        // the block's view of logits rows is never used; one row keeps the view well-formed
+        s << block_arena_floats() + cfg_.vocab << " create_var\n";
+        s << cfg_.batch << " " << cfg_.tokens << " create_dynamic_here\n";
+        s << "0 #  " << i << " share_batch_tensors\n";
+    }
+    s << "0 #\n";
+    return s.str();
+}
+
+std::string BloomTrainer::step_script() const {
+    std::ostringstream s;
+    const int n = cfg_.layers;
+    s << "0 # model_input\n";
+    s << "1 # 'xinput' @  0 # 'xinput' @  op.copy   1 # layer_forward\n";
+    for (int i = 2; i <= n; i++)
+        s << i << " # 'xinput' @  " << i - 1 << " # 'xa' @  op.copy   " << i << " # layer_forward\n";
+    s << "0 # 'xa' @  " << n << " # 'xa' @  op.copy   0 # model_head\n";
+    s << n << " # 'yout_g' @  0 # 'xc' @  op.copy   " << n << " # layer_backward_core\n";
+    for (int i = n - 1; i >= 1; i--)
+        s << i << " # 'yout_g' @  " << i + 1 << " # 'xa' @  op.copy   " << i << " # layer_backward_core\n";
+    s << "0 # 'xb' @  1 # 'xa' @  op.copy   0 # model_input_backward\n";
+    s << "op.sync\n";
+    return s.str();
+}
+
+void BloomTrainer::create() {
+    env_.execute(setup_script());
+    step_.reset(env_.build(step_script()));
+}
+
+void BloomTrainer::init_synthetic(uint64_t seed, float std) {
+    std::ostringstream s;
+    s.precision(9);
+    auto matrix = [&](const char* name, uint64_t sd) {
+        s << "'" << name << "' @ 0 " << std << " " << sd << " bloom.normal\n";
+    };
+    s << "0 #\n";
+    matrix("word_embeddings.weight", seed * 1000003ull);
+    s << "'word_embeddings_layernorm.weight' @ 1 op.fill  'word_embeddings_layernorm.bias' @ op.zero\n";
+    s << "'ln_f.weight' @ 1 op.fill  'ln_f.bias' @ op.zero\n";
+    for (int i = 1; i <= cfg_.layers; i++) {
+        const uint64_t base = (seed + (uint64_t)i) * 1000003ull;
+        s << i << " #\n";
+        matrix("query_key_value.weight", base + 1);
+        matrix("dense.weight", base + 2);
+        matrix("dense_h_to_4h.weight", base + 3);
+        matrix("dense_4h_to_h.weight", base + 4);
+        s << "'input_layernorm.weight' @ 1 op.fill  'input_layernorm.bias' @ op.zero\n";
+        s << "'post_attention_layernorm.weight' @ 1 op.fill  'post_attention_layernorm.bias' @ op.zero\n";
+        s << "'query_key_value.bias' @ op.zero  'dense.bias' @ op.zero\n";
+        s << "'dense_h_to_4h.bias' @ op.zero  'dense_4h_to_h.bias' @ op.zero\n";
+    }
+    s << "0 # op.sync\n";
+    env_.execute(s.str());
+}
+
+float BloomTrainer::step(const int32_t* ids, const int32_t* mask) {
+    br_assert(step_ != nullptr, "BloomTrainer::create has not run");
+    env_.change(0);
+    const size_t n = (size_t)(cfg_.batch * cfg_.tokens);
+    tensor_t t_ids = env_.hash().find_tensor("ids_");
+    tensor_t t_mask = env_.hash().find_tensor("mask_");
+    memcpy(t_ids->data(), ids, n * sizeof(int32_t));
+    memcpy(t_mask->data(), mask, n * sizeof(int32_t));
+    env_.run(step_.get());
+    return ComputingContext::last_loss;
+}
+
+}  // namespace br

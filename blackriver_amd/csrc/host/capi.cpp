@@ -6,6 +6,7 @@
 #include <memory>
 
 #include "bloom_input.hpp"
+#include "bloom_trainer.hpp"
 #include "br_hip.h"
 #include "runtime.hpp"
 #include "tensor.hpp"
@@ -17,6 +18,7 @@ using namespace br;
 struct br_env {
     std::unique_ptr<Enviroment> env;
     std::vector<std::unique_ptr<DaG>> programs;
+    std::unique_ptr<BloomTrainer> trainer;
 };
 
 namespace {
@@ -98,6 +100,7 @@ br_env_t* br_env_create(int hashes) {
 void br_env_destroy(br_env_t* e) {
     if (!e) return;
     guarded([&]() {
+        e->trainer.reset();
         e->programs.clear();
         e->env.reset();
     });
@@ -241,6 +244,39 @@ int br_env_tensor_read_i32(br_env_t* e, const char* name, int32_t* dst, int64_t 
         br_assert(t->is_cpu() && t->dtype() == DataType::Int, "tensor_read_i32: not a cpu int tensor");
         br_assert((int64_t)t->items() >= n, "tensor_read_i32: too many elements");
         memcpy(dst, t->data(), (size_t)n * sizeof(int32_t));
+    });
+}
+
+int br_bloom_model_create(br_env_t* e, int layers, int64_t batch, int64_t tokens, int64_t hidden, int64_t heads,
+                          int64_t vocab, float eps, const char* weight_dtype, const char* gemm_precision) {
+    return guarded([&]() {
+        BloomModelConfig cfg;
+        cfg.layers = layers;
+        cfg.batch = batch;
+        cfg.tokens = tokens;
+        cfg.hidden = hidden;
+        cfg.heads = heads;
+        cfg.vocab = vocab;
+        cfg.eps = eps;
+        cfg.weight_dtype = weight_dtype ? weight_dtype : "f16";
+        cfg.gemm_precision = gemm_precision ? gemm_precision : "f16";
+        e->trainer.reset(new BloomTrainer(*e->env, cfg));
+        e->trainer->create();
+    });
+}
+
+int br_bloom_model_init(br_env_t* e, uint64_t seed, float std) {
+    return guarded([&]() {
+        br_assert(e->trainer != nullptr, "br_bloom_model_create has not run");
+        e->trainer->init_synthetic(seed, std);
+    });
+}
+
+int br_bloom_model_step(br_env_t* e, const int32_t* ids, const int32_t* mask, float* loss) {
+    return guarded([&]() {
+        br_assert(e->trainer != nullptr, "br_bloom_model_create has not run");
+        const float l = e->trainer->step(ids, mask);
+        if (loss) *loss = l;
     });
 }
 

@@ -458,12 +458,24 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
                           code(lm_head), hidden, 0, 0, logits, BR_F32, vocab, 0, nullptr, 1, compute));
         BR_OP(br_hip_logsoftmax_nll_fwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, d_logp + r0, d_result, rows,
                                         vocab, stream()));
-        BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, logits, BR_F32, scale, rows,
-                                        vocab, stream()));
-        BR_OP(product(0, 0, rows, hidden, vocab, 1.0f, logits, BR_F32, vocab, 0, lm_head->data(), code(lm_head),
-                          hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute));
-        BR_OP(product(1, 0, vocab, hidden, rows, 1.0f, logits, BR_F32, vocab, 0, x + r0 * hidden, BR_F32, hidden,
-                          0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
+        // dlogits: written as fp16 straight away when the products run in fp16
+        // (the same rounding the GEMM would apply to an fp32 copy), else fp32
+        // in place and converted once for the two products below
+        Operand dl{logits, BR_F32};
+        if (compute == BR_GEMM_F16 && (rows * vocab) % 8 == 0) {
+            void* dl16 = ComputingContext::gemm_staging(1, (size_t)(rows * vocab) * 2);
+            BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, dl16, BR_F16, scale, rows,
+                                            vocab, stream()));
+            dl = Operand{dl16, BR_F16};
+        } else {
+            BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, logits, BR_F32, scale,
+                                            rows, vocab, stream()));
+            dl = shared_operand(logits, BR_F32, rows * vocab, compute);
+        }
+        BR_OP(product(0, 0, rows, hidden, vocab, 1.0f, dl.ptr, dl.dtype, vocab, 0, lm_head->data(), code(lm_head),
+                      hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute));
+        BR_OP(product(1, 0, vocab, hidden, rows, 1.0f, dl.ptr, dl.dtype, vocab, 0, x + r0 * hidden, BR_F32, hidden,
+                      0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
     }
 
     // sum of log p(label) in fp64 on the host, as the reference accumulates it
@@ -489,6 +501,7 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
     }
 
     const float ret = count > 0 ? (float)(total / (double)count) : 0.0f;
+    ComputingContext::last_loss = ret;
     std::cout << "#################  " << count << " " << ret << std::endl;
     return ret;
 }

@@ -25,6 +25,9 @@ struct ComputingContext {
     // MFMA type used when every operand of a product is stored as fp32:
     // BR_GEMM_F32 (default, fp32-faithful), BR_GEMM_F16 or BR_GEMM_BF16.
     static int fp32_gemm_compute;
+    // what the most recent op_loss_backward returned (the word leaves nothing
+    // on the stack; drivers read the value here)
+    static float last_loss;
 
     static void boot(int dev);  // 128 MiB of scratch like context.cpp:31
     static void shutdown();

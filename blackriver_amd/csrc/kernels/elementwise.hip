@@ -578,6 +578,29 @@ __global__ __launch_bounds__(kBlock) void xmask_table_kernel(const int32_t* mask
 
 bool fits_u32(int64_t v) { return v > 0 && v <= 0xffffffffLL; }
 
+// ---------------------------------------------------------- normal fill
+// dst[i] = mean + std * z_i with z_i a standard normal that depends only on
+// (seed, i): SplitMix64 of the pair gives two 24-bit uniforms, Box-Muller one
+// normal.  The same (seed, i) gives the same value on any launch geometry.
+__device__ __forceinline__ unsigned long long splitmix64(unsigned long long x) {
+    x += 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    return x ^ (x >> 31);
+}
+template <typename T>
+__global__ __launch_bounds__(kBlock) void normal_kernel(T* dst, float mean, float std, unsigned long long seed,
+                                                         int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        const unsigned long long h = splitmix64(splitmix64(seed) ^ (unsigned long long)i);
+        const float u1 = ((float)(unsigned)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
+        const float u2 = (float)(unsigned)((h >> 8) & 0xffffffu) * (1.0f / 16777216.0f);
+        const float z = sqrtf(-2.0f * __logf(u1)) * __cosf(6.28318530718f * u2);
+        dst[i] = from_f32<T>(mean + std * z);
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -595,6 +618,24 @@ int br_hip_fill(void* dst, int dtype, float value, int64_t n, br_stream_t stream
             fill_kernel<__hip_bfloat16><<<grid, kBlock, 0, st>>>((__hip_bfloat16*)dst, __float2bfloat16(value), n);
             break;
         case BR_I32: fill_kernel<int32_t><<<grid, kBlock, 0, st>>>((int32_t*)dst, (int32_t)value, n); break;
+        default: return BR_ERR_TODO;
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_normal(void* dst, int dtype, float mean, float std, uint64_t seed, int64_t n, br_stream_t stream) {
+    if (n < 0) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!dst) return BR_ERR_OUTPUT;
+    hipStream_t st = as_stream(stream);
+    const int grid = grid_for(n, kBlock);
+    switch (dtype) {
+        case BR_F32: normal_kernel<float><<<grid, kBlock, 0, st>>>((float*)dst, mean, std, seed, n); break;
+        case BR_F16: normal_kernel<__half><<<grid, kBlock, 0, st>>>((__half*)dst, mean, std, seed, n); break;
+        case BR_BF16:
+            normal_kernel<__hip_bfloat16><<<grid, kBlock, 0, st>>>((__hip_bfloat16*)dst, mean, std, seed, n);
+            break;
         default: return BR_ERR_TODO;
     }
     BR_HIP_LAUNCH_CHECK();

@@ -44,6 +44,7 @@ SIGNATURES = {
     "br_hip_memcpy_d2d": (_int, [_vp, _vp, _sz, _vp]),
     "br_hip_memset": (_int, [_vp, _int, _sz, _vp]),
     "br_hip_fill": (_int, [_vp, _int, _f32, _i64, _vp]),
+    "br_hip_normal": (_int, [_vp, _int, _f32, _f32, ctypes.c_uint64, _i64, _vp]),
     "br_hip_cast": (_int, [_vp, _int, _vp, _int, _i64, _vp]),
     "br_hip_add_bcast": (_int, [_vp, _vp, _vp, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), _vp]),
     "br_hip_gelu_fwd": (_int, [_vp, _vp, _int, _i64, _vp]),

@@ -50,6 +50,9 @@ SIGNATURES = {
     "br_env_tensor_read": (_int, [_vp, _cp, _f32p, _i64]),
     "br_env_tensor_write_i32": (_int, [_vp, _cp, _i32p, _i64]),
     "br_env_tensor_read_i32": (_int, [_vp, _cp, _i32p, _i64]),
+    "br_bloom_model_create": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _i64, ctypes.c_float, _cp, _cp]),
+    "br_bloom_model_init": (_int, [_vp, ctypes.c_uint64, ctypes.c_float]),
+    "br_bloom_model_step": (_int, [_vp, _i32p, _i32p, ctypes.POINTER(ctypes.c_float)]),
     "br_bloom_fetch_data": (_int, [_i32p, _i32p, _i64, _i64, _f32p, _i64, _i64, _f32p, _f32p, _f32p]),
 }
 
@@ -225,6 +228,47 @@ class Env:
             _check(self._lib.br_env_tensor_read(self._h, name.encode(), out.ctypes.data_as(_f32p), out.size),
                    "read(%s)" % name)
         return out
+
+
+class BloomModel:
+    """A whole BLOOM model on one GPU (C++ driver BloomTrainer): block i in
+    hash i of `env`, embedding / final LayerNorm / LM head in hash 0."""
+
+    def __init__(self, layers, batch, tokens, hidden=4096, heads=32, vocab=250880, eps=1e-5, weight_dtype="f16",
+                 gemm_precision="f16"):
+        self.layers, self.batch, self.tokens = layers, batch, tokens
+        self.hidden, self.heads, self.vocab, self.eps = hidden, heads, vocab, eps
+        self.env = Env(layers + 1)
+        self.env.execute(words_text("bloom.words"))
+        self.env.execute(words_text("bloom_model.words"))
+        _check(load().br_bloom_model_create(self.env._h, layers, batch, tokens, hidden, heads, vocab, eps,
+                                            weight_dtype.encode(), gemm_precision.encode()), "model_create")
+
+    def init(self, seed=0, std=0.02):
+        _check(load().br_bloom_model_init(self.env._h, seed, std), "model_init")
+
+    def step(self, ids, mask) -> float:
+        ids = np.ascontiguousarray(ids, np.int32)
+        mask = np.ascontiguousarray(mask, np.int32)
+        assert ids.shape == (self.batch, self.tokens) and mask.shape == ids.shape
+        loss = ctypes.c_float()
+        _check(load().br_bloom_model_step(self.env._h, ids.ctypes.data_as(_i32p), mask.ctypes.data_as(_i32p),
+                                          ctypes.byref(loss)), "model_step")
+        return loss.value
+
+    def read(self, layer, name):
+        self.env.change_hash(layer)
+        out = self.env.read(name)
+        self.env.change_hash(0)
+        return out
+
+    def write(self, layer, name, array):
+        self.env.change_hash(layer)
+        self.env.write(name, array)
+        self.env.change_hash(0)
+
+    def close(self):
+        self.env.close()
 
 
 def fetch_data(ids, mask, heads, vocab=None):

@@ -74,6 +74,13 @@ int br_hip_memset(void* dst, int byte_value, size_t bytes, br_stream_t stream);
 /* ---- elementwise ------------------------------------------------------- */
 /* cudnnSetTensor in cuda_tensor.cpp:111-125 (op_fill). */
 int br_hip_fill(void* dst, int dtype, float value, int64_t n, br_stream_t stream);
+/* Synthetic initialisation: dst[i] = mean + std * z(seed, i), z standard normal
+ * from a counter-based generator (SplitMix64 + Box-Muller), dtype BR_F32 /
+ * BR_F16 / BR_BF16.  No counterpart in the reference, which only ever reads
+ * weights from files (io_load, cuda_tensor.cpp:52-72); benchmarks and tests of
+ * whole models use it where those files do not exist. */
+int br_hip_normal(void* dst, int dtype, float mean, float std, uint64_t seed, int64_t n,
+                  br_stream_t stream);
 
 /* Storage conversion between BR_F32, BR_F16 and BR_BF16 (no counterpart in
  * the reference, whose only implemented dtype is fp32). */

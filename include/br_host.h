@@ -78,6 +78,22 @@ int br_env_tensor_read(br_env_t* env, const char* name, float* dst, int64_t n);
 int br_env_tensor_write_i32(br_env_t* env, const char* name, const int32_t* src, int64_t n);
 int br_env_tensor_read_i32(br_env_t* env, const char* name, int32_t* dst, int64_t n);
 
+/* Whole-model training on one GPU: the main loop of blackriver/train_bloom.cpp:123-199
+ * (create the tensors, then per step: fetch_data + run the training words)
+ * without MPI ranks and host weight streaming.  `env` needs layers + 1 hashes
+ * and must already have executed bloom.words and bloom_model.words.  Block i
+ * lives in hash i (weights, fp32 gradients, its own activation arena), the
+ * embedding / final LayerNorm / LM head in hash 0.
+ *   create: allocates everything and compiles the step program
+ *   init:   N(0, std) matrices, unit LayerNorm scales, zero biases
+ *   step:   ids / mask are [batch, tokens] int32 host arrays; *loss receives
+ *           what op.loss_backward returns (mean log-probability of the labels) */
+int br_bloom_model_create(br_env_t* env, int layers, int64_t batch, int64_t tokens, int64_t hidden,
+                          int64_t heads, int64_t vocab, float eps, const char* weight_dtype,
+                          const char* gemm_precision);
+int br_bloom_model_init(br_env_t* env, uint64_t seed, float std);
+int br_bloom_model_step(br_env_t* env, const int32_t* ids, const int32_t* mask, float* loss);
+
 /* The host-side batch preparation of BloomInput::fetch_data
  * (train_bloom.cpp:41-93) on caller-provided host buffers:
  *   xinput[i,:] = vocab[ids[i],:]             (when vocab != NULL)
