@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the BLOOM-7B1 training hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--leg all|block|roofline|elementwise|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--leg all|block|model|roofline|elementwise|copy]
 
 A "step" is one forward + backward pass of one BLOOM-7B1 decoder block
 (hidden 4096, 32 heads x 128, FFN 16384, ALiBi causal attention, batch 4 x
@@ -52,7 +52,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--leg", default="all", choices=["all", "block", "roofline", "elementwise", "copy"])
+    ap.add_argument("--leg", default="all", choices=["all", "block", "model", "roofline", "elementwise", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     return ap.parse_args()
 
@@ -118,6 +118,30 @@ def block_leg(args, host, hip, timer):
     assert np.all(np.isfinite(out)), "block step produced non-finite values"
     env.close()
     return sec
+
+
+def model_leg(args, host, timer):
+    """BASELINE configs[4]: 30 blocks + embedding LayerNorm + final LayerNorm +
+    LM-head loss, forward and backward, batch 1 x 512, every layer resident."""
+    layers, batch, tokens = 30, 1, T
+    model = host.BloomModel(layers, batch, tokens, H, NH, V, 1e-5, "f16", "f16")
+    model.init(4, 0.02)
+    rng = np.random.default_rng(4)
+    ids = rng.integers(0, V, (batch, tokens)).astype(np.int32)
+    mask = np.ones((batch, tokens), np.int32)
+    mask[0, tokens - 37:] = 0                       # right padding, 37 of 512 masked
+    steps = max(3, args.steps // 4)
+    losses = []
+    sec = timer.run(lambda i: losses.append(model.step(ids, mask)), steps, 2)
+    assert all(np.isfinite(l) for l in losses), "model step produced a non-finite loss"
+    n = batch * tokens
+    fwd_block = 2.0 * n * H * (3 * H + H + 2 * F) + 2 * 2.0 * batch * NH * tokens * tokens * (H // NH)
+    flop = 3.0 * (layers * fwd_block + 2.0 * n * H * V)
+    model.close()
+    return {"workload": "BLOOM-7B1, 30 blocks + LM head (BASELINE configs[4]), batch 1 x 512, fp16 weights, "
+                        "no recomputation", "ms_per_step": sec * 1e3, "tokens_per_s": n / sec,
+            "gemm_tflop_per_step": flop / 1e12, "gemm_tflops": flop / sec / 1e12, "loss": losses[-1],
+            "steps": steps}
 
 
 def gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch=1, iters=20, staged=False):
@@ -295,6 +319,7 @@ def main():
         sys.exit(2)
     torch.cuda.init()
     host.boot(0, 1 << 30)
+    host.set_echo_loss(False)   # stdout carries the one JSON line
     stream = ctypes.c_void_p(host.stream())
     timer = Timer(hip, stream)
     timer.device_sync = torch.cuda.synchronize
@@ -313,6 +338,8 @@ def main():
         result["ms_per_step"] = sec * 1e3
         result["step_gemm_tflops"] = STEP_GEMM_FLOP / sec / 1e12
         result["step_frac_of_mfma_peak"] = STEP_GEMM_FLOP / sec / 1e12 / MFMA_F16_PEAK_TFLOPS
+    if args.leg in ("all", "model"):
+        result["model"] = model_leg(args, host, timer)
     if args.leg in ("all", "roofline"):
         roof, gemms = roofline_leg(hip, timer, torch, full=args.leg == "all")
         result["roofline"] = roof

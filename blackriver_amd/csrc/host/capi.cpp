@@ -84,6 +84,11 @@ int br_host_set_fp32_gemm_compute(int compute) {
     return 0;
 }
 
+int br_host_set_echo_loss(int on) {
+    ComputingContext::echo_loss = on != 0;
+    return 0;
+}
+
 br_env_t* br_env_create(int hashes) {
     br_env_t* e = new br_env();
     if (guarded([&]() {

@@ -502,7 +502,7 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
 
     const float ret = count > 0 ? (float)(total / (double)count) : 0.0f;
     ComputingContext::last_loss = ret;
-    std::cout << "#################  " << count << " " << ret << std::endl;
+    if (ComputingContext::echo_loss) std::cout << "#################  " << count << " " << ret << std::endl;
     return ret;
 }
 

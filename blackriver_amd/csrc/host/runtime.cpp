@@ -53,6 +53,7 @@ void* ComputingContext::host_workspace = nullptr;
 size_t ComputingContext::workspace_size = 0;
 int ComputingContext::fp32_gemm_compute = BR_GEMM_F32;
 float ComputingContext::last_loss = 0.0f;
+bool ComputingContext::echo_loss = true;
 void* ComputingContext::scratch_ptr_ = nullptr;
 size_t ComputingContext::scratch_size_ = 0;
 void* ComputingContext::staging_ptr_[2] = {nullptr, nullptr};

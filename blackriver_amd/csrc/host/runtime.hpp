@@ -28,6 +28,9 @@ struct ComputingContext {
     // what the most recent op_loss_backward returned (the word leaves nothing
     // on the stack; drivers read the value here)
     static float last_loss;
+    // op_loss_backward prints "#################  <count> <loss>" like the
+    // reference (cuda_tensor.cpp:692) unless a driver turns it off
+    static bool echo_loss;
 
     static void boot(int dev);  // 128 MiB of scratch like context.cpp:31
     static void shutdown();

@@ -50,6 +50,7 @@ SIGNATURES = {
     "br_env_tensor_read": (_int, [_vp, _cp, _f32p, _i64]),
     "br_env_tensor_write_i32": (_int, [_vp, _cp, _i32p, _i64]),
     "br_env_tensor_read_i32": (_int, [_vp, _cp, _i32p, _i64]),
+    "br_host_set_echo_loss": (_int, [_int]),
     "br_bloom_model_create": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _i64, ctypes.c_float, _cp, _cp]),
     "br_bloom_model_init": (_int, [_vp, ctypes.c_uint64, ctypes.c_float]),
     "br_bloom_model_step": (_int, [_vp, _i32p, _i32p, ctypes.POINTER(ctypes.c_float)]),
@@ -111,6 +112,11 @@ def stream():
 
 def sync() -> None:
     _check(load().br_host_sync(), "br_host_sync")
+
+
+def set_echo_loss(on: bool) -> None:
+    """Whether op.loss_backward prints its '#################  count loss' line."""
+    load().br_host_set_echo_loss(1 if on else 0)
 
 
 def words_text(name: str) -> str:

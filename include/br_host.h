@@ -38,6 +38,10 @@ void* br_host_stream(void);
 int br_host_sync(void);
 /* BR_GEMM_F16 / BR_GEMM_BF16 / BR_GEMM_F32 for products of fp32-stored operands. */
 int br_host_set_fp32_gemm_compute(int compute);
+/* op.loss_backward prints "#################  <count> <loss>" on stdout as the
+ * reference does (cuda_tensor.cpp:692); 0 turns that off for drivers that own
+ * stdout. */
+int br_host_set_echo_loss(int on);
 
 /* An Enviroment with `hashes` namespaces and the io.* / op.* words loaded
  * (train_bloom.cpp:125-126). */
