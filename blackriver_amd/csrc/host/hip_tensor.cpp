@@ -60,14 +60,15 @@ constexpr size_t kTailBytes = 8u << 20;
 char* tail() { return static_cast<char*>(ComputingContext::workspace) + ComputingContext::workspace_size - kTailBytes; }
 size_t head_bytes() { return ComputingContext::workspace_size - kTailBytes; }
 
-// Every matrix product of the backend.  With a 16-bit MFMA type, fp32 operands
-// are staged as 16-bit copies first (br_hip_gemm_staged), which lets the
-// product run on the direct-to-LDS kernel; fp32 compute goes straight through.
+// Every matrix product of the backend.  With a 16-bit MFMA type the product
+// goes through br_hip_gemm_staged: fp32 operands are staged as 16-bit copies
+// first, which lets the product run on the direct-to-LDS kernel, and products
+// with few output tiles are split along K; fp32 compute goes straight through.
 int product(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a, int a_dtype,
             int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb, int64_t stride_b, int accumulate,
             void* c, int c_dtype, int64_t ldc, int64_t stride_c, const float* bias, int64_t batch, int compute) {
     void* stream = ComputingContext::stream;
-    if (compute == BR_GEMM_F32 || (a_dtype != BR_F32 && b_dtype != BR_F32))
+    if (compute == BR_GEMM_F32)
         return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
                            accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
     const size_t need = br_hip_gemm_staged_workspace(trans_a, trans_b, m, n, k, a_dtype, b_dtype, batch);

@@ -18,7 +18,7 @@
 #include <stdlib.h>
 #include <string.h>
 
-#include "gemm_mfma16.hpp"
+#include "gemm_dtl16.hpp"
 
 using namespace brk;
 
@@ -335,6 +335,69 @@ int stage_rows(const float* src, long long ld, long long stride, long long rows,
     return BR_OK;
 }
 
+// ---- split-K ------------------------------------------------------------------
+// A product with few output tiles and a long K leaves most CUs idle.  It is run
+// as a strided-batched product over `splits` slices of K into fp32 partials
+// (slice s of A / B is the operand advanced by s * k/splits along k, which the
+// batch strides express), followed by a fixed-order sum: deterministic, no
+// atomics.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4* __restrict__ part, int splits,
+                                                            long long mn4, long long n4, float alpha,
+                                                            const float* __restrict__ bias, int accumulate,
+                                                            void* __restrict__ c, int c_dtype, long long ldc) {
+    for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < mn4;
+         i += (long long)gridDim.x * blockDim.x) {
+        float4 s = part[i];
+        for (int p = 1; p < splits; p++) {
+            const float4 v = part[(long long)p * mn4 + i];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        const long long row = i / n4, col = (i % n4) * 4;
+        float o[4] = {alpha * s.x, alpha * s.y, alpha * s.z, alpha * s.w};
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] += bias[col + j];
+        }
+        if (c_dtype == BR_F32) {
+            float* dst = static_cast<float*>(c) + row * ldc + col;
+#pragma unroll
+            for (int j = 0; j < 4; j++) dst[j] = accumulate ? o[j] + dst[j] : o[j];
+        } else if (c_dtype == BR_F16) {
+            __half* dst = static_cast<__half*>(c) + row * ldc + col;
+#pragma unroll
+            for (int j = 0; j < 4; j++) dst[j] = __float2half_rn(accumulate ? o[j] + __half2float(dst[j]) : o[j]);
+        } else {
+            __hip_bfloat16* dst = static_cast<__hip_bfloat16*>(c) + row * ldc + col;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                dst[j] = __float2bfloat16(accumulate ? o[j] + __bfloat162float(dst[j]) : o[j]);
+        }
+    }
+}
+
+// Number of K slices (1 = do not split) for an unbatched product on the
+// direct-to-LDS kernel: the split whose estimated time, including the pass
+// over the partials, is smallest.
+int splitk_choice(int64_t m, int64_t n, int64_t k) {
+    if (n % 4 != 0) return 1;
+    double best = gemm16::dtl_plan(m, n, k, 1).seconds;
+    int pick = 1;
+    for (int s = 2; s <= 16; s *= 2) {
+        if (k % (64 * s) != 0 || k / s < 512) break;
+        const double t = gemm16::dtl_plan(m, n, k / s, s).seconds + 6e-6 + (double)(s + 1) * m * n * 4.0 / 4e12;
+        if (t < 0.85 * best) {
+            best = t;
+            pick = s;
+        }
+    }
+    static const char* force = getenv("BR_GEMM_SPLITK");
+    if (force) {
+        const int f = atoi(force);
+        if (f >= 1 && k % (64 * f) == 0) pick = f;
+    }
+    return pick;
+}
+
 size_t staged_bytes(int64_t rows, int64_t cols, int64_t batch) {
     const size_t b = (size_t)rows * (size_t)cols * (size_t)batch * 2;
     return (b + 255) & ~(size_t)255;
@@ -350,6 +413,10 @@ extern "C" size_t br_hip_gemm_staged_workspace(int trans_a, int trans_b, int64_t
     size_t need = 0;
     if (a_dtype == BR_F32) need += staged_bytes(m, k, batch);
     if (b_dtype == BR_F32) need += staged_bytes(k, n, batch);
+    if (batch == 1) {
+        const int splits = splitk_choice(m, n, k);
+        if (splits > 1) need += (size_t)splits * (size_t)m * (size_t)n * sizeof(float);
+    }
     return need;
 }
 
@@ -360,12 +427,13 @@ extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n
                                   size_t workspace_bytes, br_stream_t stream) {
     const bool f32_a = a_dtype == BR_F32, f32_b = b_dtype == BR_F32;
     const bool sixteen = compute == BR_GEMM_F16 || compute == BR_GEMM_BF16;
-    // Stage only when the converted problem meets the direct-to-LDS kernel's
-    // rules; every other case is the plain entry point's business.
+    // Stage (and consider splitting K) only when the converted problem meets the
+    // direct-to-LDS kernel's rules; every other case is the plain entry point's
+    // business.
     const int64_t a_rows = trans_a ? k : m, a_cols = trans_a ? m : k;
     const int64_t b_rows = trans_b ? n : k, b_cols = trans_b ? k : n;
-    bool stage = sixteen && (f32_a || f32_b) && workspace && aligned16(workspace) && m > 0 && n > 0 && k > 0 &&
-                 batch > 0 && a && b && k % 32 == 0;
+    bool stage = sixteen && workspace && aligned16(workspace) && m > 0 && n > 0 && k > 0 && batch > 0 && a && b &&
+                 k % 32 == 0;
     if (stage) {
         // dense 16-bit copies: leading dimension = cols, batch stride = rows*cols
         if (f32_a && a_cols % 8 != 0) stage = false;
@@ -396,6 +464,24 @@ extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n
         b_dtype = native;
         ldb = b_cols;
         stride_b = b_rows * b_cols;
+        ws += staged_bytes(k, n, batch);
+    }
+    const int splits = batch == 1 ? splitk_choice(m, n, k) : 1;
+    if (splits > 1 && c) {
+        // slices of K as batch entries: a k-contiguous operand advances by k/splits
+        // elements per slice, a row-contiguous one by k/splits rows
+        const int64_t ks = k / splits;
+        float* part = reinterpret_cast<float*>(ws);
+        const int rc = br_hip_gemm(trans_a, trans_b, m, n, ks, 1.0f, a, a_dtype, lda, trans_a ? ks * lda : ks, b,
+                                   b_dtype, ldb, trans_b ? ks : ks * ldb, 0, part, BR_F32, n, m * n, nullptr, splits,
+                                   compute, stream);
+        if (rc != BR_OK) return rc;
+        const long long mn4 = m * n / 4;
+        splitk_reduce_kernel<<<grid_for(mn4, 256, 1 << 14), 256, 0, st>>>(reinterpret_cast<const float4*>(part),
+                                                                        splits, mn4, n / 4, alpha, bias,
+                                                                        accumulate ? 1 : 0, c, c_dtype, ldc);
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
     }
     return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
                        accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);

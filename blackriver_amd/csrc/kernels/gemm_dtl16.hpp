@@ -321,28 +321,42 @@ inline bool dtl_applies(const GemmArgs& g, const Problem& p) {
     return a_span < lim && b_span < lim;
 }
 
-// Tile choice: estimated time = rounds of workgroups over the 256 CUs x tile
-// area / relative MFMA rate of the configuration (measured on the BLOOM-7B1
-// linear-layer shapes: 256x256 ~ 1.0, 256x128 ~ 0.9, 128x128 ~ 0.8 with two
-// workgroups resident per CU).
+// Tile choice by estimated time: rounds of workgroups over the 256 CUs x the
+// MFMA work of one tile / the rate a workgroup of that configuration reaches
+// (measured on the BLOOM-7B1 linear-layer shapes: ~1000 TFLOP/s chip-wide for
+// 256x256, ~0.9 of that for 256x128, ~0.8 for 128x128 with two workgroups
+// resident per CU).
+struct DtlPlan {
+    int config;      // 0: 256x256, 1: 256x128, 2: 128x128 (64-wide K steps), 3: 128x128 with 32-wide steps
+    double seconds;  // estimate, for comparing plans only
+};
+inline DtlPlan dtl_plan(long long m, long long n, long long k, long long batch) {
+    const double per_cu = 1.0e15 / 256.0;  // flop/s of one CU at the 256x256 rate
+    auto estimate = [&](long long bm, long long bn, long long slots, double rel) {
+        const long long tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch;
+        const double rounds = (double)((tiles + slots - 1) / slots);
+        const double per_block = per_cu * rel * 256.0 / (double)slots;  // co-resident workgroups share the CU
+        return rounds * 2.0 * (double)bm * (double)bn * (double)k / per_block + 4e-6;
+    };
+    if (k % 64 != 0) return DtlPlan{3, estimate(128, 128, 512, 0.65)};
+    DtlPlan best{0, estimate(256, 256, 256, 1.0)};
+    const double t1 = estimate(256, 128, 256, 0.9), t2 = estimate(128, 128, 512, 0.8);
+    if (t1 < best.seconds) best = DtlPlan{1, t1};
+    if (t2 < best.seconds) best = DtlPlan{2, t2};
+    return best;
+}
+
 template <int CT>
 int launch_dtl(const GemmArgs& g, const Problem& p, long long batch, hipStream_t st) {
-    if (g.k % 64 != 0) return launch_dtl_config<CT, 128, 128, 64, 64, 32, 3>(g, p, batch, st);
-    auto rounds = [&](long long bm, long long bn, long long slots) {
-        const long long tiles = ((g.m + bm - 1) / bm) * ((g.n + bn - 1) / bn) * batch;
-        return (double)((tiles + slots - 1) / slots);
-    };
-    const double c256 = rounds(256, 256, 256) * 256 * 256 / 1.0;
-    const double c256x128 = rounds(256, 128, 256) * 256 * 128 / 0.9;
-    const double c128 = rounds(128, 128, 512) * 2 * 128 * 128 / 0.8;
+    int pick = dtl_plan(g.m, g.n, g.k, batch).config;
     static const char* force = getenv("BR_GEMM_TILE");
-    int pick = c256 <= c256x128 && c256 <= c128 ? 0 : (c256x128 <= c128 ? 1 : 2);
-    if (force && strcmp(force, "256x256") == 0) pick = 0;
-    if (force && strcmp(force, "256x128") == 0) pick = 1;
-    if (force && strcmp(force, "128x128") == 0) pick = 2;
+    if (pick != 3 && force && strcmp(force, "256x256") == 0) pick = 0;
+    if (pick != 3 && force && strcmp(force, "256x128") == 0) pick = 1;
+    if (pick != 3 && force && strcmp(force, "128x128") == 0) pick = 2;
     if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
     if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
-    return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
+    if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
+    return launch_dtl_config<CT, 128, 128, 64, 64, 32, 3>(g, p, batch, st);
 }
 
 template <int CT>

@@ -221,12 +221,15 @@ int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float
  * copies, one pass each), so that the product runs on the direct-to-LDS
  * kernel that needs both operands in the MFMA type.  Replaces the same
  * kernels::LtSgemm call (LtSgemm.cu:55-126); `workspace` plays the part of
- * the scratch the reference hands to cublasLtMatmul (context.cpp:31).  Falls back to br_hip_gemm when `compute`
+ * the scratch the reference hands to cublasLtMatmul (context.cpp:31).  An
+ * unbatched product with too few output tiles for the 256 CUs and a long K is
+ * split along K into fp32 partials in the same workspace and summed in a fixed
+ * order (deterministic).  Falls back to br_hip_gemm when `compute`
  * is BR_GEMM_F32, no operand is fp32, the shape is not 16-byte friendly
  * (k % 32, operand row lengths % 8) or the workspace is smaller than
- * br_hip_gemm_staged_workspace() bytes.  Results are identical to
- * br_hip_gemm's for the same `compute` (same rounding of the operands, same
- * accumulation order within a tile configuration). */
+ * br_hip_gemm_staged_workspace() bytes.  Results equal br_hip_gemm's for the
+ * same `compute` up to the order of the fp32 summation (same rounding of the
+ * operands). */
 size_t br_hip_gemm_staged_workspace(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
                                     int a_dtype, int b_dtype, int64_t batch);
 int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,

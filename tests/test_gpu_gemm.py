@@ -208,6 +208,36 @@ def test_gemm_staged_matches_plain_entry(ta, tb, a_dt, b_dt):
     assert_close(staged, plain, 1e-5, "staged vs plain")
 
 
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("a_dt,b_dt,c_dt", [(F32, F16, F32), (F16, F16, F16), (F32, F32, F32)])
+def test_gemm_staged_split_k(ta, tb, a_dt, b_dt, c_dt):
+    """Few output tiles and a long K: the staged entry splits K (the workspace
+    figure shows it) and must still give the plain product, with alpha, bias
+    and accumulation applied once."""
+    rng = np.random.default_rng(10)
+    m, n, k = 256, 384, 4096
+    print("case split-k ta=%d tb=%d dtypes=%s" % (ta, tb, (a_dt, b_dt, c_dt)), flush=True)
+    a, b = operands(rng, ta, tb, m, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c0 = rng.standard_normal((1, m, n)).astype(np.float32)
+    da, db_, dbias = to_dev(a, a_dt), to_dev(b, b_dt), dev(bias)
+    need = hip.load().br_hip_gemm_staged_workspace(int(ta), int(tb), m, n, k, a_dt, b_dt, 1)
+    copies = sum(2 * r * c for r, c, dt in ((m, k, a_dt), (k, n, b_dt)) if dt == F32)
+    splits = (need - copies) // (4 * m * n)
+    assert splits >= 2 and need == copies + splits * 4 * m * n
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    c = to_dev(c0, c_dt)
+    call("br_hip_gemm_staged", int(ta), int(tb), m, n, k, 0.5, ptr(da), a_dt, m if ta else k, 0, ptr(db_), b_dt,
+         k if tb else n, 0, 1, ptr(c), c_dt, n, 0, ptr(dbias), 1, hip.GEMM_F16, ptr(ws), need, stream())
+    A = to_host64(da).reshape((k, m) if ta else (m, k))
+    B = to_host64(db_).reshape((n, k) if tb else (k, n))
+    ref = 0.5 * ((A.T if ta else A) @ (B.T if tb else B)) + bias.astype(np.float64)[None, :] + \
+        to_host64(to_dev(c0, c_dt)).reshape(m, n)
+    assert_close(to_host64(c).reshape(m, n), ref, 2e-2, "split-k staged gemm")
+    if c_dt == F32:
+        assert np.sqrt(np.mean((to_host64(c).reshape(m, n) - ref) ** 2)) < 1e-3 * np.sqrt(np.mean(ref ** 2))
+
+
 def test_gemm_staged_falls_back():
     rng = np.random.default_rng(9)
     # K not a multiple of 32, fp32 compute, and a workspace that is too small
