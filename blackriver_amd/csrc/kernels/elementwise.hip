@@ -192,23 +192,26 @@ __global__ __launch_bounds__(kBlock) void add_bcast_scalar(const T* a, const T* 
 // ------------------------------------------------------------------ GELU
 // gelu(v) = v * (0.5 + 0.5*tanh(u)),  u = v*(0.79788456 + 0.03567741 v^2)
 //         = v * sigmoid(2u)            (no cancellation in the left tail)
+// sigmoid(2u) = 1 / (1 + 2^w), w = -2*log2(e)*u: the factor is folded into the
+// two polynomial constants, so the exponent costs no extra multiplies.
+constexpr float kLog2e2 = 2.8853900817779268f;  // 2 * log2(e)
 __device__ __forceinline__ float gelu_one(float v) {
-    const float u = v * (0.79788456f + 0.03567741f * v * v);
-    return v * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
+    const float w = v * (-kLog2e2 * 0.79788456f + (-kLog2e2 * 0.03567741f) * (v * v));
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(w));
 }
 
 // d/dv gelu(v) = s + 2 v s (1 - s) u',  s = sigmoid(2u),
 //   u = 0.79788456 v (1 + 0.044715 v^2),  u' = 0.79788456 + 0.1070322243 v^2
-// evaluated from e = exp(-2|u|) in (0,1] so that s and s(1-s) keep full
-// relative accuracy for large |v|.
+// evaluated from e = exp(-2|u|) = 2^(-|w|), w = 2*log2(e)*u, in (0,1] so that s
+// and s(1-s) keep full relative accuracy for large |v|.
 __device__ __forceinline__ float gelu_grad_one(float v) {
     const float v2 = v * v;
-    const float u = 0.79788456f * v * (1.0f + 0.044715f * v2);
-    const float e = __expf(-2.0f * fabsf(u));
+    const float w = v * (kLog2e2 * 0.79788456f + (kLog2e2 * 0.79788456f * 0.044715f) * v2);
+    const float e = __builtin_amdgcn_exp2f(-fabsf(w));
     const float inv = __builtin_amdgcn_rcpf(1.0f + e);
-    const float s = u >= 0.f ? inv : e * inv;
-    const float s1ms = e * inv * inv;
-    return s + 2.0f * v * s1ms * (0.79788456f + 0.1070322243f * v2);
+    const float ei = e * inv;
+    const float s = w >= 0.f ? inv : ei;
+    return s + v * (ei * inv) * (2.0f * 0.79788456f + (2.0f * 0.1070322243f) * v2);
 }
 
 __global__ __launch_bounds__(kBlock) void gelu_fwd_f32(const float* x, float* y, int64_t n4) {
@@ -319,7 +322,20 @@ __global__ __launch_bounds__(kBlock) void bias_gelu_fwd_kernel(const T* x, const
     for (int j = 0; j < VEC; j++) b[j] = bias[col + j];
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
     const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
-    for (int64_t r = r0; r < r1; r++) {
+    // four rows of loads in flight per thread
+    int64_t r = r0;
+    for (; r + 4 <= r1; r += 4) {
+        float v[4][VEC];
+#pragma unroll
+        for (int u = 0; u < 4; u++) VecIO<T, VEC>::load(x + (r + u) * cols + col, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) v[u][j] = gelu_one(v[u][j] + b[j]);
+            VecIO<T, VEC>::store(y + (r + u) * cols + col, v[u]);
+        }
+    }
+    for (; r < r1; r++) {
         float v[VEC];
         VecIO<T, VEC>::load(x + r * cols + col, v);
 #pragma unroll
@@ -342,15 +358,31 @@ __global__ __launch_bounds__(kBlock) void bias_gelu_bwd_kernel(const T* dy, cons
     }
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
     const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
-    for (int64_t r = r0; r < r1; r++) {
+    // two rows (four loads) in flight per thread; rows are still summed in order
+    int64_t r = r0;
+    for (; r + 2 <= r1; r += 2) {
+        float v[2][VEC], g[2][VEC];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            VecIO<T, VEC>::load(x + (r + u) * cols + col, v[u]);
+            VecIO<T, VEC>::load(dy + (r + u) * cols + col, g[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) g[u][j] *= gelu_grad_one(v[u][j] + b[j]);
+            // sum what was stored, i.e. after rounding to the storage type
+            VecIO<T, VEC>::store_rounded(dx + (r + u) * cols + col, g[u]);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[j] += g[u][j];
+        }
+    }
+    for (; r < r1; r++) {
         float v[VEC], g[VEC];
         VecIO<T, VEC>::load(x + r * cols + col, v);
         VecIO<T, VEC>::load(dy + r * cols + col, g);
 #pragma unroll
-        for (int j = 0; j < VEC; j++) {
-            g[j] *= gelu_grad_one(v[j] + b[j]);
-        }
-        // sum what was stored, i.e. after rounding to the storage type
+        for (int j = 0; j < VEC; j++) g[j] *= gelu_grad_one(v[j] + b[j]);
         VecIO<T, VEC>::store_rounded(dx + r * cols + col, g);
 #pragma unroll
         for (int j = 0; j < VEC; j++) acc[j] += g[j];
