@@ -130,10 +130,23 @@ int br_env_run(br_env_t* e, int program) {
     });
 }
 
+namespace {
+int disassemble_into(br_env_t* e, const char* text, bool fused, char* out, size_t out_bytes);
+}
+
 int br_env_disassemble(br_env_t* e, const char* text, char* out, size_t out_bytes) {
+    return disassemble_into(e, text, false, out, out_bytes);
+}
+
+int br_env_disassemble_fused(br_env_t* e, const char* text, char* out, size_t out_bytes) {
+    return disassemble_into(e, text, true, out, out_bytes);
+}
+
+namespace {
+int disassemble_into(br_env_t* e, const char* text, bool fused, char* out, size_t out_bytes) {
     std::string joined;
     const int rc = guarded([&]() {
-        for (const std::string& s : e->env->disassemble(text)) {
+        for (const std::string& s : e->env->disassemble(text, fused)) {
             joined += s;
             joined += '\n';
         }
@@ -143,6 +156,7 @@ int br_env_disassemble(br_env_t* e, const char* text, char* out, size_t out_byte
     memcpy(out, joined.c_str(), joined.size() + 1);
     return 0;
 }
+}  // namespace
 
 int br_env_change_hash(br_env_t* e, int hash) {
     return guarded([&]() { e->env->change((size_t)hash); });

@@ -309,6 +309,7 @@ void Enviroment::run_(DaG* dag) {
             case DaG::Step::PushString: stack_.push_string(s.str); break;
             case DaG::Step::RunBuiltin: dag->builtins_[s.idx]->run(this); break;
             case DaG::Step::RunNative: dag->natives_[s.idx]->run(stack_); break;
+            case DaG::Step::Skip: break;
             default: br_panic("Runing binary error can't bere!");
         }
     }
@@ -324,10 +325,48 @@ void Enviroment::insert_native_word(const std::string& name, NativeCreator* fn) 
     native_words_[name] = fn;
 }
 
+void Enviroment::insert_fusion(const std::vector<std::string>& sequence, const std::string& fused) {
+    br_assert(sequence.size() >= 2, "a fusion needs at least two words");
+    br_assert(native_words_.count(fused) != 0, "the fused word must be registered first");
+    fusions_.emplace_back(sequence, fused);
+}
+
+// Peephole pass over a linked program (see insert_fusion).
+void Enviroment::fuse(DaG& dag) {
+    auto is_push = [](const DaG::Step& s) {
+        return s.kind == DaG::Step::PushString || (s.kind == DaG::Step::RunBuiltin && s.str == "@");
+    };
+    for (const auto& fusion : fusions_) {
+        const std::vector<std::string>& seq = fusion.first;
+        for (size_t i = 0; i < dag.steps_.size(); i++) {
+            if (dag.steps_[i].kind != DaG::Step::RunNative || dag.steps_[i].str != seq[0]) continue;
+            std::vector<size_t> at{i};
+            size_t pc = i + 1;
+            while (at.size() < seq.size() && pc < dag.steps_.size()) {
+                const DaG::Step& s = dag.steps_[pc];
+                if (s.kind == DaG::Step::RunNative && s.str == seq[at.size()]) {
+                    at.push_back(pc);
+                } else if (!is_push(s)) {
+                    break;
+                }
+                pc++;
+            }
+            if (at.size() != seq.size()) continue;
+            for (size_t k = 0; k + 1 < at.size(); k++) dag.steps_[at[k]].kind = DaG::Step::Skip;
+            DaG::Step& last = dag.steps_[at.back()];
+            last.str = fusion.second;
+            last.idx = dag.natives_.size();
+            dag.natives_.push_back(native_words_[fusion.second](*this));
+            i = at.back();
+        }
+    }
+}
+
 DaG* Enviroment::build(const std::string& txt) {
     std::unique_ptr<DaG> dag(new DaG(this));
     UserWord code = compile(txt);
     linking(*dag, code);
+    fuse(*dag);
     return dag.release();
 }
 
@@ -340,13 +379,15 @@ void Enviroment::execute(const std::string& txt) {
     DaG dag(this);
     UserWord code = compile(txt);
     linking(dag, code);
+    fuse(dag);
     run_(&dag);
 }
 
-std::vector<std::string> Enviroment::disassemble(const std::string& txt) {
+std::vector<std::string> Enviroment::disassemble(const std::string& txt, bool fused) {
     DaG dag(this);
     UserWord code = compile(txt);
     linking(dag, code);
+    if (fused) fuse(dag);
     std::vector<std::string> out;
     for (const DaG::Step& s : dag.steps_) {
         std::ostringstream ss;
@@ -355,6 +396,7 @@ std::vector<std::string> Enviroment::disassemble(const std::string& txt) {
             case DaG::Step::PushString: ss << "S:" << s.str; break;
             case DaG::Step::RunBuiltin: ss << "B:" << s.str; break;
             case DaG::Step::RunNative: ss << "W:" << s.str; break;
+            case DaG::Step::Skip: ss << "-:" << s.str; break;
         }
         out.push_back(ss.str());
     }

@@ -198,7 +198,7 @@ struct DaG {
 
 private:
     struct Step {
-        enum Kind { PushNumber, PushString, RunBuiltin, RunNative } kind;
+        enum Kind { PushNumber, PushString, RunBuiltin, RunNative, Skip } kind;
         double num;
         std::string str;
         size_t idx;
@@ -215,6 +215,13 @@ struct Enviroment {
     ~Enviroment() {}
 
     void insert_native_word(const std::string& name, NativeCreator* fn);
+    // Registers a fusion: wherever a linked program runs the native words
+    // `sequence` one after the other with nothing but operand pushes
+    // (strings and `@`) in between, the earlier words are skipped -- their
+    // operands simply stay on the stack -- and the last one is replaced by
+    // `fused`, which pops the operands of the whole sequence (first word's
+    // deepest) and must produce exactly what the sequence would have.
+    void insert_fusion(const std::vector<std::string>& sequence, const std::string& fused);
 
     // compile + link; the caller owns the result and runs it with run()
     DaG* build(const std::string& txt);
@@ -222,8 +229,11 @@ struct Enviroment {
     // compile + link + run once
     void execute(const std::string& txt);
     // compile + link, then list the flat program one step per entry:
-    // "N:<number>", "S:<string>", "B:<builtin>", "W:<native word>"
-    std::vector<std::string> disassemble(const std::string& txt);
+    // "N:<number>", "S:<string>", "B:<builtin>", "W:<native word>"; with
+    // `fused` the program is listed after the fusion pass that build() and
+    // execute() apply ("-:<native word>" marks a word whose work moved into
+    // the fused word that follows)
+    std::vector<std::string> disassemble(const std::string& txt, bool fused = false);
 
     Stack& stack() { return stack_; }
     Hash& hash() { return hashes_[target_]; }
@@ -234,11 +244,13 @@ struct Enviroment {
 private:
     UserWord compile(const std::string& txt);
     void linking(DaG& dag, UserWord& word);
+    void fuse(DaG& dag);
     void run_(DaG* dag);
     void load_base_words();
 
     std::map<std::string, UserWord> user_words_;
     std::map<std::string, NativeCreator*> native_words_;
+    std::vector<std::pair<std::vector<std::string>, std::string>> fusions_;
     Stack stack_;
     std::vector<Hash> hashes_;
     size_t target_;

@@ -91,6 +91,38 @@ BR_WORD(QueryKey, Tensors<3> a(stack); a[0]->op_qk(a[0], a[1], a[2]);)
 BR_WORD(Add, Tensors<3> a(stack); a[0]->op_add(a[0], a[1], a[2]);)
 // ( x out -- )
 BR_WORD(Softmax, Tensors<2> a(stack); a[0]->op_softmax(a[0], a[1]);)
+// ( s alibi s  s xmask s  s p -- )  the operands of `op.add op.add op.softmax`
+// as bloomz-7b/train.words:158-162 strings them together on the attention
+// scores.  When they have that shape (one fp32 device tensor [B,NH,T,T] updated
+// in place, alibi [1,NH,1,T], xmask [B,1,T,T]) the three passes run as one
+// kernel that applies the same operations in the same order (bit-identical);
+// anything else runs the three operators one after the other.
+BR_WORD(AddAddSoftmax,
+    Tensors<8> a(stack);
+    auto same = [](const tensor_t& x, const tensor_t& y) { return x->data() == y->data() && x->items() == y->items(); };
+    auto f32dev = [](const tensor_t& x) { return x->is_cuda() && x->dtype() == DataType::Float; };
+    bool fast = f32dev(a[0]) && f32dev(a[1]) && f32dev(a[4]) && f32dev(a[7]) && a[0]->shape().dim() == 4 &&
+                a[1]->shape().dim() == 4 && a[4]->shape().dim() == 4 && same(a[0], a[2]) && same(a[0], a[3]) &&
+                same(a[0], a[5]) && same(a[0], a[6]) && a[7]->items() == a[0]->items();
+    if (fast) {
+        const auto& xs = a[0]->shape();
+        const auto& as = a[1]->shape();
+        const auto& ms = a[4]->shape();
+        fast = as[0] == 1 && as[1] == xs[1] && as[2] == 1 && as[3] == xs[3] && ms[0] == xs[0] && ms[1] == 1 &&
+               ms[2] == xs[2] && ms[3] == xs[3];
+        if (fast) {
+            BR_HIP_CHECK(br_hip_alibi_masked_softmax_fwd(
+                static_cast<const float*>(a[0]->data()), static_cast<const float*>(a[1]->data()),
+                static_cast<const float*>(a[4]->data()), static_cast<float*>(a[7]->data()), (int64_t)xs[0],
+                (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], ComputingContext::stream));
+        }
+    }
+    if (!fast) {
+        a[0]->op_add(a[0], a[1], a[2]);
+        a[3]->op_add(a[3], a[4], a[5]);
+        a[6]->op_softmax(a[6], a[7]);
+    }
+)
 // ( p v out -- )
 BR_WORD(Attn, Tensors<3> a(stack); a[0]->op_attn(a[0], a[1], a[2]);)
 // ( x out -- )
@@ -155,6 +187,7 @@ void load_nn_words(Enviroment& env) {
         {"op.add", Add::creator},
         {"op.querykey", QueryKey::creator},
         {"op.softmax", Softmax::creator},
+        {"op.add_add_softmax", AddAddSoftmax::creator},
         {"op.attn", Attn::creator},
         {"op.gelu", Gelu::creator},
         {"op.last_logits", LastLogits::creator},
@@ -168,6 +201,7 @@ void load_nn_words(Enviroment& env) {
         {"op.qk_backward", QueryKeyBackward::creator},
     };
     for (const auto& e : table) env.insert_native_word(e.name, e.creator);
+    env.insert_fusion({"op.add", "op.add", "op.softmax"}, "op.add_add_softmax");
 }
 
 }  // namespace br

@@ -35,6 +35,7 @@ SIGNATURES = {
     "br_env_execute": (_int, [_vp, _cp]),
     "br_env_build": (_int, [_vp, _cp, _ip]),
     "br_env_run": (_int, [_vp, _int]),
+    "br_env_disassemble_fused": (_int, [_vp, _cp, ctypes.c_char_p, ctypes.c_size_t]),
     "br_env_change_hash": (_int, [_vp, _int]),
     "br_env_current_hash": (_int, [_vp]),
     "br_env_set_number": (_int, [_vp, _cp, ctypes.c_double]),
@@ -192,12 +193,14 @@ class Env:
         _check(self._lib.br_env_stack_pop_number(self._h, ctypes.byref(v)), "pop_number")
         return v.value
 
-    def disassemble(self, text: str) -> list:
-        """Compile and link `text`; return the flat step list as strings."""
+    def disassemble(self, text: str, fused: bool = False) -> list:
+        """Compile and link `text`; return the flat step list as strings
+        (after the fusion pass when `fused`)."""
         size = 1 << 20
+        fn = self._lib.br_env_disassemble_fused if fused else self._lib.br_env_disassemble
         while True:
             buf = ctypes.create_string_buffer(size)
-            rc = self._lib.br_env_disassemble(self._h, text.encode(), buf, size)
+            rc = fn(self._h, text.encode(), buf, size)
             if rc == -2:
                 size *= 4
                 continue

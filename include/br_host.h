@@ -59,6 +59,10 @@ int br_env_run(br_env_t* env, int program);
  * one step per line ("N:<number>", "S:<string>", "B:<builtin>",
  * "W:<native word>"), into out.  Returns -2 when out_bytes is too small. */
 int br_env_disassemble(br_env_t* env, const char* text, char* out, size_t out_bytes);
+/* The same listing after the fusion pass that build / execute apply to a linked
+ * program ("-:<word>" marks a word whose work moved into the fused word that
+ * follows it). */
+int br_env_disassemble_fused(br_env_t* env, const char* text, char* out, size_t out_bytes);
 
 int br_env_change_hash(br_env_t* env, int hash);
 int br_env_current_hash(br_env_t* env);

@@ -169,3 +169,54 @@ def test_logsoftmax_nll_headline_shape_properties_and_sampled_rows():
     lg = host(logits[torch.arange(rows, device="cuda"), target.long()])
     want = float(((lg.astype(np.float64) - host(lse).astype(np.float64)) * (k != 0)).sum() / count)
     assert abs(r[0] - want) <= RTOL * abs(want)
+
+
+def test_fused_add_add_softmax_word_is_bit_identical_to_the_three_words(runtime):
+    """The word machine fuses `op.add op.add op.softmax`; the fused word must
+    give exactly what the three words give (each run as its own program, which
+    the fusion pass cannot see across), on the attention-score pattern and, via
+    its fallback, on operands that do not have that pattern."""
+    from blackriver_amd import host
+    rng = np.random.default_rng(12)
+    b, h, t = 2, 4, 96
+    s = rng.standard_normal((b, h, t, t)).astype(np.float32)
+    alibi = rng.standard_normal((1, h, 1, t)).astype(np.float32)
+    xmask = np.where(rng.random((b, 1, t, t)) < 0.3, -3.4028234663852886e38, 0.0).astype(np.float32)
+    env = host.Env(1)
+    try:
+        env.execute("%d %d %d %d 4 'cuda' 'float' op.create 's' !  %d %d %d %d 4 'cuda' 'float' op.create 'p' !"
+                    % (b, h, t, t, b, h, t, t))
+        env.execute("1 %d 1 %d 4 'cuda' 'float' op.create 'a' !  %d 1 %d %d 4 'cuda' 'float' op.create 'm' !"
+                    % (h, t, b, t, t))
+        env.write("a", alibi)
+        env.write("m", xmask)
+        three = ["'s' @ 'a' @ 's' @ op.add", "'s' @ 'm' @ 's' @ op.add", "'s' @ 'p' @ op.softmax"]
+        env.write("s", s)
+        for w in three:
+            env.execute(w)
+        p_separate, s_separate = env.read("p"), env.read("s")
+        env.write("s", s)
+        env.execute("  ".join(three))
+        assert np.array_equal(env.read("p"), p_separate)
+        # in place, as the model script does it
+        env.write("s", s)
+        for w in three[:2] + ["'s' @ 's' @ op.softmax"]:
+            env.execute(w)
+        in_place = env.read("s")
+        env.write("s", s)
+        env.execute("  ".join(three[:2] + ["'s' @ 's' @ op.softmax"]))
+        assert np.array_equal(env.read("s"), in_place)
+        assert np.array_equal(in_place, p_separate) and s_separate.shape == s.shape
+        # operands without the pattern (second add not in place): the fused word falls back
+        env.execute("%d %d %d %d 4 'cuda' 'float' op.create 'q' !" % (b, h, t, t))
+        other = ["'s' @ 'a' @ 's' @ op.add", "'s' @ 'm' @ 'q' @ op.add", "'q' @ 'p' @ op.softmax"]
+        env.write("s", s)
+        for w in other:
+            env.execute(w)
+        expect_p, expect_q = env.read("p"), env.read("q")
+        env.write("s", s)
+        env.execute("'p' @ op.zero 'q' @ op.zero")
+        env.execute("  ".join(other))
+        assert np.array_equal(env.read("p"), expect_p) and np.array_equal(env.read("q"), expect_q)
+    finally:
+        env.close()

@@ -169,3 +169,24 @@ def test_single_process_transport_shims(env):
     assert (env.read("m") == 3).all()
     with pytest.raises(host.HostError, match="mpi_recv"):   # nothing was sent
         env.execute("'m' @ 1 io.mpi.recv")
+
+
+def test_fusion_pass_rewrites_only_push_separated_sequences(env):
+    """`op.add op.add op.softmax` with nothing but operand pushes in between
+    becomes two skipped words and the fused word; anything else is untouched,
+    and the plain listing never changes."""
+    seq = "'s' @ 'a' @ 's' @ op.add  's' @ 'm' @ 's' @ op.add  's' @ 'p' @ op.softmax"
+    plain = env.disassemble(seq)
+    fused = env.disassemble(seq, fused=True)
+    assert [x for x in plain if x.startswith("W:")] == ["W:op.add", "W:op.add", "W:op.softmax"]
+    assert [x for x in fused if x[0] in "W-"] == ["-:op.add", "-:op.add", "W:op.add_add_softmax"]
+    assert [x for x in fused if x[0] not in "W-"] == [x for x in plain if x[0] != "W"]
+    # a number push, a hash switch or another word in between breaks the pattern
+    for middle in ("1 drop", "0 #", "op.sync"):
+        broken = seq.replace("op.add  's' @ 'm'", "op.add " + middle + " 's' @ 'm'", 1)
+        assert env.disassemble(broken, fused=True) == env.disassemble(broken)
+    # two sequences in one program are both rewritten
+    assert env.disassemble(seq + " " + seq, fused=True).count("W:op.add_add_softmax") == 2
+    # a lone add followed by softmax is not a match
+    short = "'s' @ 'm' @ 's' @ op.add  's' @ 'p' @ op.softmax"
+    assert env.disassemble(short, fused=True) == env.disassemble(short)
