@@ -24,6 +24,12 @@ int64_t BloomTrainer::block_arena_floats() const {
            cfg_.batch * cfg_.tokens * cfg_.tokens + cfg_.batch * cfg_.heads * cfg_.tokens * cfg_.tokens;
 }
 
+// 16-bit weights multiplied in their own type: product-only activations can
+// live in 16-bit operand buffers (same bits out, fewer conversions).
+bool BloomTrainer::mixed() const {
+    return cfg_.weight_dtype == cfg_.gemm_precision && (cfg_.weight_dtype == "f16");
+}
+
 int64_t BloomTrainer::model_arena_floats() const {
     // plus one logits row per position: the loss head then needs a single group
     return block_arena_floats() + cfg_.batch * cfg_.tokens * cfg_.vocab;
@@ -49,6 +55,7 @@ std::string BloomTrainer::setup_script() const {
         // the block's view of logits rows is never used; one row keeps the view well-formed
         s << block_arena_floats() + cfg_.vocab << " create_var\n";
         s << cfg_.batch << " " << cfg_.tokens << " create_dynamic_here\n";
+        if (mixed()) s << "create_operand_buffers\n";
         s << "0 #  " << i << " share_batch_tensors\n";
     }
     s << "0 #\n";
@@ -58,14 +65,16 @@ std::string BloomTrainer::setup_script() const {
 std::string BloomTrainer::step_script() const {
     std::ostringstream s;
     const int n = cfg_.layers;
+    const char* forward = mixed() ? "layer_forward_mixed" : "layer_forward";
+    const char* backward = mixed() ? "layer_backward_mixed" : "layer_backward_core";
     s << "0 # model_input\n";
-    s << "1 # 'xinput' @  0 # 'xinput' @  op.copy   1 # layer_forward\n";
+    s << "1 # 'xinput' @  0 # 'xinput' @  op.copy   1 # " << forward << "\n";
     for (int i = 2; i <= n; i++)
-        s << i << " # 'xinput' @  " << i - 1 << " # 'xa' @  op.copy   " << i << " # layer_forward\n";
+        s << i << " # 'xinput' @  " << i - 1 << " # 'xa' @  op.copy   " << i << " # " << forward << "\n";
     s << "0 # 'xa' @  " << n << " # 'xa' @  op.copy   0 # model_head\n";
-    s << n << " # 'yout_g' @  0 # 'xc' @  op.copy   " << n << " # layer_backward_core\n";
+    s << n << " # 'yout_g' @  0 # 'xc' @  op.copy   " << n << " # " << backward << "\n";
     for (int i = n - 1; i >= 1; i--)
-        s << i << " # 'yout_g' @  " << i + 1 << " # 'xa' @  op.copy   " << i << " # layer_backward_core\n";
+        s << i << " # 'yout_g' @  " << i + 1 << " # 'xa' @  op.copy   " << i << " # " << backward << "\n";
     s << "0 # 'xb' @  1 # 'xa' @  op.copy   0 # model_input_backward\n";
     s << "op.sync\n";
     return s.str();

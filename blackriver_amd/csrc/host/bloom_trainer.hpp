@@ -43,6 +43,7 @@ public:
     // floats of a block's arena / of hash 0's arena (which ends in the logits rows)
     int64_t block_arena_floats() const;
     int64_t model_arena_floats() const;
+    bool mixed() const;
     std::string setup_script() const;
     std::string step_script() const;
 

@@ -342,7 +342,14 @@ ComputingReturn HIPTensor<DT>::op_attn(tensor_t self, tensor_t v, tensor_t attn)
 template <DataType DT>
 ComputingReturn HIPTensor<DT>::op_gelu(tensor_t self, tensor_t dst) {
     if (DT == DataType::BF16) return OP_TODO_ERROR;
-    if (!dev(dst) || dst->dtype() != DT || dst->items() != self->items()) return OP_OUTPUT_ERROR;
+    if (!dev(dst) || dst->items() != self->items()) return OP_OUTPUT_ERROR;
+    if (DT == DataType::Float && dst->dtype() == DataType::F16) {
+        // fp32 activation in, fp16 operand buffer out
+        BR_OP(br_hip_gelu_fwd_f32_to_f16(static_cast<const float*>(mem_), dst->data(), (int64_t)self->items(),
+                                         stream()));
+        return OP_OK;
+    }
+    if (dst->dtype() != DT) return OP_OUTPUT_ERROR;
     BR_OP(br_hip_gelu_fwd(mem_, dst->data(), (int)DT, (int64_t)self->items(), stream()));
     return OP_OK;
 }
@@ -589,10 +596,11 @@ ComputingReturn HIPTensor<DT>::op_attn_backward(tensor_t self, tensor_t attn, te
     if (!dev(attn_g) || !dev(v_g) || attn_g->items() != attn->items() || v_g->items() != v->items())
         return OP_OUTPUT_ERROR;
     const int compute = pick_compute({self, attn, v});
-    BR_OP(product(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, mem_, (int)DT, d.hd,
-                      d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute));
-    BR_OP(product(0, 1, d.t, d.t, d.hd, 1.0f, mem_, (int)DT, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
-                      d.t * d.hd, 0, attn_g->data(), code(attn_g), d.t, d.t * d.t, nullptr, d.bh, compute));
+    const Operand d_o = shared_operand(mem_, (int)DT, d.bh * d.t * d.hd, compute);
+    BR_OP(product(1, 0, d.t, d.hd, d.t, 1.0f, attn->data(), code(attn), d.t, d.t * d.t, d_o.ptr, d_o.dtype, d.hd,
+                  d.t * d.hd, 0, v_g->data(), code(v_g), d.hd, d.t * d.hd, nullptr, d.bh, compute));
+    BR_OP(product(0, 1, d.t, d.t, d.hd, 1.0f, d_o.ptr, d_o.dtype, d.hd, d.t * d.hd, v->data(), code(v), d.hd,
+                  d.t * d.hd, 0, attn_g->data(), code(attn_g), d.t, d.t * d.t, nullptr, d.bh, compute));
     return OP_OK;
 }
 

@@ -234,6 +234,19 @@ __global__ __launch_bounds__(kBlock) void gelu_fwd_f16(const half8* x, half8* y,
     }
 }
 
+// fp32 in, fp16 out: the output of the 4h activation when it only feeds the
+// next product (rounded once, exactly as that product would round an fp32 copy)
+__global__ __launch_bounds__(kBlock) void gelu_fwd_f32_to_f16(const float4* x, half8* y, int64_t n8) {
+    const int64_t stride = (int64_t)gridDim.x * kBlock;
+    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += stride) {
+        const float4 a = x[2 * i], b = x[2 * i + 1];
+        float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int j = 0; j < 8; j++) f[j] = gelu_one(f[j]);
+        y[i] = pack8(f);
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void gelu_bwd_f32(const float* dy, const float* x, float* dx,
                                                         int64_t n4) {
     const int64_t stride = (int64_t)gridDim.x * kBlock;
@@ -747,6 +760,17 @@ static int strip_rows(int64_t rows) {
     int64_t rpb = (rows + 63) / 64;
     if (rpb < 8) rpb = 8;
     return (int)rpb;
+}
+
+int br_hip_gelu_fwd_f32_to_f16(const float* x, void* y, int64_t n, br_stream_t stream) {
+    if (n < 0) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!x) return BR_ERR_INPUT;
+    if (!y) return BR_ERR_OUTPUT;
+    if (n % 8 != 0 || !aligned16(x) || !aligned16(y)) return BR_ERR_TODO;
+    gelu_fwd_f32_to_f16<<<grid_for(n / 8, kBlock), kBlock, 0, as_stream(stream)>>>((const float4*)x, (half8*)y, n / 8);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
 }
 
 int br_hip_gelu_fwd(const void* x, void* y, int dtype, int64_t n, br_stream_t stream) {

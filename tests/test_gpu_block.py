@@ -102,6 +102,31 @@ def test_block_step_is_repeatable(runtime):
     env.close()
 
 
+@pytest.mark.parametrize("hidden,heads,batch,tokens", [(256, 4, 2, 24), (1024, 8, 2, 128)])
+def test_operand_buffer_words_give_the_same_bits(runtime, hidden, heads, batch, tokens):
+    """layer_forward_mixed / layer_backward_mixed keep product-only operands in
+    fp16 buffers; since a product rounds its fp32 operands to fp16 the same way,
+    every output and gradient must equal the fp32-arena words' bit for bit."""
+    env, w, x, dy, mask, _ = setup_block(runtime, hidden, heads, batch, tokens, "f16")
+    env.execute("create_operand_buffers")
+    env.execute("block_step op.sync")
+    names = ["xa", "xattn_in", "x4a", "xll", "input_ln_var", "post_ln_var"] + [n + "_g" for n in blk.WEIGHT_NAMES
+                                                                              if not n.startswith(("query.", "key.", "value."))]
+    names += ["query_key_value.weight_g", "query_key_value.bias_g"]
+    plain = {n: env.read(n) for n in names}
+    for n in names:
+        if n.endswith("_g"):
+            env.execute("'%s' @ op.zero" % n)
+    env.write("yout_g", dy)
+    env.write("xinput", x)
+    env.execute("block_step_mixed op.sync")
+    for n in names:
+        assert np.array_equal(env.read(n), plain[n]), n
+    # the buffers hold what the fp32 tensors round to
+    assert np.array_equal(env.read("xattn_in.h"), env.read("xattn_in").astype(np.float16).astype(np.float32))
+    env.close()
+
+
 @pytest.mark.parametrize("mode", ["fp32", "f16"])
 def test_loss_head_against_oracle(runtime, mode):
     hidden, heads, batch, tokens, vocab = 256, 4, 2, 24, 1536
