@@ -184,6 +184,16 @@ def roofline_leg(hip, timer, torch, full):
             "shape": "m=%d n=%d k=%d" % (N, F, H), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, "us_per_launch": sec * 1e6,
             "traffic": ROOFLINE_TRAFFIC_BYTES}
+    # what a bare MFMA loop (no memory traffic) reaches on this box with operands of zeros and of random values
+    scratch = torch.empty(1 << 17, device="cuda")
+    loop = {}
+    for name, rnd in (("zeros", 0), ("random", 1)):
+        tf = ctypes.c_double()
+        hip.call("br_hip_probe_mfma_f16", rnd, 8000, ctypes.c_void_p(scratch.data_ptr()), scratch.numel(),
+                 ctypes.byref(tf), timer.stream)
+        loop[name] = round(tf.value, 1)
+    roof["mfma_loop_tflops"] = loop
+    roof["frac_of_random_operand_loop"] = roof["achieved"] / loop["random"]
     gemms = []
     if full:
         hd = H // NH
