@@ -553,9 +553,19 @@ ComputingReturn HIPTensor<DT>::op_linear_backward(tensor_t self, tensor_t x, ten
     if (DT == DataType::BF16) return OP_TODO_ERROR;
     const size_t need = br_hip_colsum_workspace(n, out);
     void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
-    BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, ws, need, stream()));
+    Operand dy{mem_, (int)DT};
+    if (DT == DataType::Float && compute != BR_GEMM_F32 && out % 8 == 0) {
+        // one pass over dy: its column sums and the 16-bit copy both products read
+        const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
+        void* dy16 = ComputingContext::gemm_staging(1, (size_t)(n * out) * 2);
+        BR_OP(br_hip_colsum_cast(static_cast<const float*>(mem_), static_cast<float*>(bias_g->data()), dy16, native, n,
+                                 out, ws, need, stream()));
+        dy = Operand{dy16, native};
+    } else {
+        BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, ws, need, stream()));
+        dy = shared_operand(mem_, (int)DT, n * out, compute);
+    }
     // weight_g[out,in] = dy^T . x
-    const Operand dy = shared_operand(mem_, (int)DT, n * out, compute);
     BR_OP(product(1, 0, out, in, n, 1.0f, dy.ptr, dy.dtype, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
                   code(weight_g), in, 0, nullptr, 1, compute));
     // x_g[n,in] = dy . W

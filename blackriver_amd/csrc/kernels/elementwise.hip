@@ -463,6 +463,48 @@ __global__ __launch_bounds__(kBlock) void colsum_partial_vec(const T* __restrict
     for (int j = 0; j < VEC; j++) partial[(int64_t)blockIdx.y * cols + col + j] = acc[j];
 }
 
+// Stage 1 for fp32 x that is also wanted as a 16-bit copy (the gradient of a
+// linear layer: its column sums are the bias gradient, its 16-bit copy is the
+// operand of the two products that follow): one pass over x does both.
+template <typename D>
+__global__ __launch_bounds__(kBlock) void colsum_cast_partial(const float* __restrict__ x, float* __restrict__ partial,
+                                                               D* __restrict__ x16, int64_t rows, int64_t cols,
+                                                               int rows_per_block) {
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * 4;
+    if (col >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    auto emit = [&](int64_t r, const float (&v)[4]) {
+        const unsigned lo = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[0])) |
+                            ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[1])) << 16);
+        const unsigned hi = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[2])) |
+                            ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[3])) << 16);
+        *reinterpret_cast<uint2*>(x16 + r * cols + col) = make_uint2(lo, hi);
+    };
+    int64_t r = r0;
+    for (; r + 4 <= r1; r += 4) {
+        float v[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) VecIO<float, 4>::load(x + (r + u) * cols + col, v[u]);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[j] += v[u][j];
+            emit(r + u, v[u]);
+        }
+    }
+    for (; r < r1; r++) {
+        float v[4];
+        VecIO<float, 4>::load(x + r * cols + col, v);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] += v[j];
+        emit(r, v);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) partial[(int64_t)blockIdx.y * cols + col + j] = acc[j];
+}
+
 // Stage 2 for cols % 4 == 0: 1024 threads = 16 column quads x 64 slices of
 // groups, every load of a workgroup in flight at once; slices are combined in
 // LDS in a fixed order.
@@ -937,6 +979,28 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
         colsum_partial<float><<<grid, kBlock, 0, st>>>((const float*)x, partial, rows, cols, rpb);
     else
         colsum_partial<__half><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
+    BR_HIP_LAUNCH_CHECK();
+    return colsum_finish(partial, out, groups, cols, st);
+}
+
+int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int64_t rows, int64_t cols,
+                       void* workspace, size_t workspace_bytes, br_stream_t stream) {
+    if (rows <= 0 || cols <= 0) return BR_ERR_ATTR;
+    if (!x) return BR_ERR_INPUT;
+    if (!out || !x16) return BR_ERR_OUTPUT;
+    if (x16_dtype != BR_F16 && x16_dtype != BR_BF16) return BR_ERR_TODO;
+    if (cols % 4 != 0 || !aligned16(x) || (reinterpret_cast<uintptr_t>(x16) & 7u) != 0) return BR_ERR_TODO;
+    if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
+    hipStream_t st = as_stream(stream);
+    float* partial = (float*)workspace;
+    const int64_t blocks_x = (cols / 4 + kBlock - 1) / kBlock;
+    const int rpb = colsum_vec_rows_per_block(rows, blocks_x);
+    const int groups = (int)((rows + rpb - 1) / rpb);
+    dim3 grid((unsigned)blocks_x, (unsigned)groups);
+    if (x16_dtype == BR_F16)
+        colsum_cast_partial<__half><<<grid, kBlock, 0, st>>>(x, partial, (__half*)x16, rows, cols, rpb);
+    else
+        colsum_cast_partial<__hip_bfloat16><<<grid, kBlock, 0, st>>>(x, partial, (__hip_bfloat16*)x16, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
     return colsum_finish(partial, out, groups, cols, st);
 }

@@ -128,6 +128,13 @@ int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, in
 size_t br_hip_colsum_workspace(int64_t rows, int64_t cols);
 int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols,
                   void* workspace, size_t workspace_bytes, br_stream_t stream);
+/* The same column sums of an fp32 x together with a 16-bit copy of x (x16,
+ * BR_F16 or BR_BF16, dense [rows, cols]) in one pass: op_linear_backward
+ * (cuda_tensor.cpp:730-812) needs the sums as the bias gradient and, with a
+ * 16-bit MFMA type, the copy as the operand of its two products.  cols % 4 == 0,
+ * x 16-byte aligned; workspace as for br_hip_colsum. */
+int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int64_t rows, int64_t cols,
+                       void* workspace, size_t workspace_bytes, br_stream_t stream);
 
 /* ---- LayerNorm --------------------------------------------------------- */
 /* kernels::launch_layer_norm_float, kernels/normalize_kernels.cu:87-102

@@ -137,6 +137,22 @@ def test_colsum(rows, cols):
     assert_close(host(out), x.astype(np.float64).sum(0), RTOL, "colsum")
 
 
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (300, 1000), (5, 8), (1, 4)])
+def test_colsum_cast_equals_colsum_plus_cast(rows, cols):
+    """One pass giving the column sums and the fp16 copy: the sums must equal
+    br_hip_colsum's bit for bit (same strips, same order), the copy the cast's."""
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    dx = dev(x)
+    ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
+    sums, sums2, h = empty(cols), empty(cols), empty((rows, cols), torch.float16)
+    call("br_hip_colsum", ptr(dx), F32, ptr(sums), rows, cols, ptr(ws), ws.numel(), stream())
+    call("br_hip_colsum_cast", ptr(dx), ptr(sums2), ptr(h), F16, rows, cols, ptr(ws), ws.numel(), stream())
+    assert np.array_equal(host(sums2), host(sums))
+    assert np.array_equal(host(h).view(np.uint16), x.astype(np.float16).view(np.uint16))
+    assert_close(host(sums2), x.astype(np.float64).sum(0), RTOL, "colsum")
+
+
 def test_fill_and_cast_roundtrip():
     n = 100003
     t = empty(n)
