@@ -301,12 +301,13 @@ def copy_leg(hip, timer, torch):
 
 def cpu_baseline_leg():
     """The CPU oracle (a restatement of the reference's operators; the
-    reference itself has no CPU math path) on a bounded sample: the same
-    block at batch 2 x 512 tokens, forward + backward, all host threads."""
+    reference itself has no CPU math path) on a bounded sample: one step of
+    the same block at the same batch 4 x 512 tokens, forward + backward, all
+    host threads (about 13 s)."""
     import oracle as orc
     from oracle import bloom_block as blk
     rng = np.random.default_rng(3)
-    b, t = 2, 512
+    b, t = B, T
     w = blk.make_weights(rng, H, std=0.02)
     x = rng.standard_normal((b, t, H)).astype(np.float32)
     dy = rng.standard_normal((b, t, H)).astype(np.float32)
@@ -316,8 +317,8 @@ def cpu_baseline_leg():
     blk.layer_backward(w, s, x, dy, NH)
     sec = time.perf_counter() - t0
     return {"value": b * t / sec, "unit": "tokens/s", "cores": orc.threads(), "kind": "port",
-            "sample": "same block (H=4096, 32 heads, FFN 16384) fwd+bwd at batch %d x %d tokens, fp32 storage with "
-                      "fp64 accumulation, %.1f s of CPU work" % (b, t, sec)}
+            "sample": "one step of the same block (H=4096, 32 heads, FFN 16384) fwd+bwd at batch %d x %d tokens, fp32 "
+                      "storage with fp64 accumulation, %.1f s of CPU work" % (b, t, sec)}
 
 
 def main():
