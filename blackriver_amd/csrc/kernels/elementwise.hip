@@ -684,7 +684,11 @@ __global__ __launch_bounds__(kBlock) void normal_kernel(T* dst, float mean, floa
         const float u1 = ((float)(unsigned)(h >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
         const float u2 = (float)(unsigned)((h >> 8) & 0xffffffu) * (1.0f / 16777216.0f);
         const float z = sqrtf(-2.0f * __logf(u1)) * __cosf(6.28318530718f * u2);
-        dst[i] = from_f32<T>(mean + std * z);
+        float value = mean + std * z;
+        // keep the fp32 rounding: without the barrier the multiply-add is fused into
+        // the 16-bit conversion and a 16-bit tensor would not be the rounded fp32 one
+        asm volatile("" : "+v"(value));
+        dst[i] = from_f32<T>(value);
     }
 }
 

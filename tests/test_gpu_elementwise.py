@@ -153,6 +153,52 @@ def test_colsum_cast_equals_colsum_plus_cast(rows, cols):
     assert_close(host(sums2), x.astype(np.float64).sum(0), RTOL, "colsum")
 
 
+def test_gelu_fwd_f32_to_f16_rounds_the_fp32_result_once():
+    rng = np.random.default_rng(9)
+    n = 8 * 4099
+    x = (2.0 * rng.standard_normal(n)).astype(np.float32)
+    dx = dev(x)
+    y32, y16 = empty(n), empty(n, torch.float16)
+    call("br_hip_gelu_fwd", ptr(dx), ptr(y32), F32, n, stream())
+    call("br_hip_gelu_fwd_f32_to_f16", ptr(dx), ptr(y16), n, stream())
+    assert np.array_equal(host(y16).view(np.uint16), host(y32).astype(np.float16).view(np.uint16))
+    lib = hip.load()
+    assert lib.br_hip_gelu_fwd_f32_to_f16(ptr(dx), ptr(y16), 12, stream()) == -1      # n % 8 != 0: not this entry's job
+    assert lib.br_hip_gelu_fwd_f32_to_f16(ptr(dx), ptr(y16), 0, stream()) == 0
+    torch.cuda.synchronize()
+
+
+def test_normal_fill_is_a_function_of_seed_and_index():
+    n = 1 << 20
+    a, b, c = empty(n), empty(n), empty(n)
+    h = empty(n, torch.float16)
+    call("br_hip_normal", ptr(a), F32, 1.0, 0.5, 7, n, stream())
+    call("br_hip_normal", ptr(b), F32, 1.0, 0.5, 7, n, stream())
+    call("br_hip_normal", ptr(c), F32, 1.0, 0.5, 8, n, stream())
+    call("br_hip_normal", ptr(h), F16, 1.0, 0.5, 7, n, stream())
+    va, vb, vc = host(a).astype(np.float64), host(b), host(c)
+    assert np.array_equal(host(a), vb) and not np.array_equal(host(a), vc)
+    assert np.array_equal(host(h).view(np.uint16), host(a).astype(np.float16).view(np.uint16))
+    # a prefix is the same whatever the length (value depends on the index only)
+    short = empty(1000)
+    call("br_hip_normal", ptr(short), F32, 1.0, 0.5, 7, 1000, stream())
+    assert np.array_equal(host(short), host(a)[:1000])
+    z = (va - 1.0) / 0.5
+    assert abs(z.mean()) < 5e-3 and abs(z.std() - 1.0) < 5e-3
+    assert abs((z ** 3).mean()) < 2e-2 and abs((z ** 4).mean() - 3.0) < 5e-2      # skewness 0, kurtosis 3
+    assert abs(np.corrcoef(z[:-1], z[1:])[0, 1]) < 5e-3                            # neighbours uncorrelated
+    assert np.all(np.isfinite(va))
+
+
+def test_mfma_probe_reports_a_rate():
+    scratch = empty(1 << 17)
+    for rnd in (0, 1):
+        tf = ctypes.c_double()
+        call("br_hip_probe_mfma_f16", rnd, 200, ptr(scratch), scratch.numel(), ctypes.byref(tf), stream())
+        assert 100.0 < tf.value < 5000.0
+    assert hip.load().br_hip_probe_mfma_f16(0, 200, ptr(scratch), 10, ctypes.byref(tf), stream()) == -4
+
+
 def test_fill_and_cast_roundtrip():
     n = 100003
     t = empty(n)
