@@ -10,6 +10,7 @@ Two modes:
 """
 import numpy as np
 import pytest
+import torch
 
 import oracle as orc
 from oracle import bloom_block as blk
@@ -25,18 +26,21 @@ def setup_block(runtime, hidden, heads, batch, tokens, mode, vocab=1024, seed=3)
     env.execute(host.words_text("bloom.words"))
     env.execute("%d %d %d 1e-05 model_dims" % (hidden, heads, vocab))
     env.set("$DEVICE", "cuda")
-    env.set("$WDTYPE", "f16" if mode == "f16" else "float")
-    env.execute("'%s' op.gemm_precision" % ("f16" if mode == "f16" else "f32"))
+    env.set("$WDTYPE", {"f16": "f16", "bf16": "bf16"}.get(mode, "float"))
+    env.execute("'%s' op.gemm_precision" % {"f16": "f16", "bf16": "bf16"}.get(mode, "f32"))
     env.execute("create_layer_weight create_layer_grad zero_layer_grad")
     env.execute("%d %d dynamic_floats" % (batch, tokens))
     floats = int(env.pop_number()) + 64 * vocab
     env.execute("%d create_var  %d %d create_dynamic" % (floats, batch, tokens))
 
     w = blk.make_weights(rng, hidden, std=0.02)
-    if mode == "f16":   # the oracle sees the weights exactly as the device stores them
+    if mode in ("f16", "bf16"):   # the oracle sees the weights exactly as the device stores them
         for k in w:
             if k.endswith(".weight") and "layernorm" not in k:
-                w[k] = w[k].astype(np.float16).astype(np.float32)
+                if mode == "f16":
+                    w[k] = w[k].astype(np.float16).astype(np.float32)
+                else:
+                    w[k] = torch.from_numpy(w[k]).to(torch.bfloat16).to(torch.float32).numpy()
     env.write("query_key_value.weight", np.concatenate([w["query.weight"], w["key.weight"], w["value.weight"]]))
     env.write("query_key_value.bias", np.concatenate([w["query.bias"], w["key.bias"], w["value.bias"]]))
     for name in blk.WEIGHT_NAMES:
@@ -60,10 +64,12 @@ def setup_block(runtime, hidden, heads, batch, tokens, mode, vocab=1024, seed=3)
     ("fp32", 1024, 8, 2, 128),
     ("f16", 256, 4, 2, 24),
     ("f16", 1024, 8, 2, 128),
+    ("bf16", 1024, 8, 2, 128),
 ])
 def test_block_forward_backward_against_oracle(runtime, mode, hidden, heads, batch, tokens):
     print("case", mode, hidden, heads, batch, tokens, flush=True)
-    tol = 1e-4 if mode == "fp32" else 2e-2
+    # bf16 multiplicands carry 8 significant bits: operand rounding alone is 4x fp16's at these magnitudes
+    tol = {"fp32": 1e-4, "f16": 2e-2, "bf16": 6e-2}[mode]
     env, w, x, dy, mask, _ = setup_block(runtime, hidden, heads, batch, tokens, mode)
     # the device-built tables are bit-exact
     assert np.array_equal(env.read("alibi").reshape(heads, tokens), orc.alibi(heads, tokens))
@@ -85,7 +91,7 @@ def test_block_forward_backward_against_oracle(runtime, mode, hidden, heads, bat
         assert_close(env.read(name + "_g").reshape(g_ref[name + "_g"].shape), g_ref[name + "_g"], tol, name + "_g")
     # key bias gradient is zero in exact arithmetic (softmax shift invariance)
     scale = float(np.sqrt(np.mean(g_ref["query.bias_g"].astype(np.float64) ** 2)))
-    assert np.max(np.abs(env.read("key.bias_g"))) < (1e-3 if mode == "fp32" else 5e-2) * scale
+    assert np.max(np.abs(env.read("key.bias_g"))) < {"fp32": 1e-3, "f16": 5e-2, "bf16": 2e-1}[mode] * scale
     env.close()
 
 
