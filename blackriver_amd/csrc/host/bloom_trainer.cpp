@@ -27,7 +27,7 @@ int64_t BloomTrainer::block_arena_floats() const {
 // 16-bit weights multiplied in their own type: product-only activations can
 // live in 16-bit operand buffers (same bits out, fewer conversions).
 bool BloomTrainer::mixed() const {
-    return cfg_.weight_dtype == cfg_.gemm_precision && (cfg_.weight_dtype == "f16");
+    return cfg_.weight_dtype == cfg_.gemm_precision && (cfg_.weight_dtype == "f16" || cfg_.weight_dtype == "bf16");
 }
 
 int64_t BloomTrainer::model_arena_floats() const {

@@ -343,10 +343,10 @@ template <DataType DT>
 ComputingReturn HIPTensor<DT>::op_gelu(tensor_t self, tensor_t dst) {
     if (DT == DataType::BF16) return OP_TODO_ERROR;
     if (!dev(dst) || dst->items() != self->items()) return OP_OUTPUT_ERROR;
-    if (DT == DataType::Float && dst->dtype() == DataType::F16) {
-        // fp32 activation in, fp16 operand buffer out
-        BR_OP(br_hip_gelu_fwd_f32_to_f16(static_cast<const float*>(mem_), dst->data(), (int64_t)self->items(),
-                                         stream()));
+    if (DT == DataType::Float && (dst->dtype() == DataType::F16 || dst->dtype() == DataType::BF16)) {
+        // fp32 activation in, 16-bit operand buffer out
+        BR_OP(br_hip_gelu_fwd_f32_to_16(static_cast<const float*>(mem_), dst->data(), code(dst), (int64_t)self->items(),
+                                        stream()));
         return OP_OK;
     }
     if (dst->dtype() != DT) return OP_OUTPUT_ERROR;

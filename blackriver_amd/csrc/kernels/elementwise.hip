@@ -234,16 +234,24 @@ __global__ __launch_bounds__(kBlock) void gelu_fwd_f16(const half8* x, half8* y,
     }
 }
 
-// fp32 in, fp16 out: the output of the 4h activation when it only feeds the
+// fp32 in, 16-bit out: the output of the 4h activation when it only feeds the
 // next product (rounded once, exactly as that product would round an fp32 copy)
-__global__ __launch_bounds__(kBlock) void gelu_fwd_f32_to_f16(const float4* x, half8* y, int64_t n8) {
+template <typename D>
+__global__ __launch_bounds__(kBlock) void gelu_fwd_f32_to_16(const float4* x, uint4* y, int64_t n8) {
     const int64_t stride = (int64_t)gridDim.x * kBlock;
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += stride) {
         const float4 a = x[2 * i], b = x[2 * i + 1];
         float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        unsigned w[4];
 #pragma unroll
-        for (int j = 0; j < 8; j++) f[j] = gelu_one(f[j]);
-        y[i] = pack8(f);
+        for (int j = 0; j < 4; j++) {
+            float lo = gelu_one(f[2 * j]), hi = gelu_one(f[2 * j + 1]);
+            // the fp32 results are rounded to fp32 first, then to the 16-bit type
+            asm volatile("" : "+v"(lo), "+v"(hi));
+            w[j] = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(lo)) |
+                   ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(hi)) << 16);
+        }
+        y[i] = make_uint4(w[0], w[1], w[2], w[3]);
     }
 }
 
@@ -808,13 +816,18 @@ static int strip_rows(int64_t rows) {
     return (int)rpb;
 }
 
-int br_hip_gelu_fwd_f32_to_f16(const float* x, void* y, int64_t n, br_stream_t stream) {
+int br_hip_gelu_fwd_f32_to_16(const float* x, void* y, int y_dtype, int64_t n, br_stream_t stream) {
     if (n < 0) return BR_ERR_ATTR;
     if (n == 0) return BR_OK;
     if (!x) return BR_ERR_INPUT;
     if (!y) return BR_ERR_OUTPUT;
+    if (y_dtype != BR_F16 && y_dtype != BR_BF16) return BR_ERR_TODO;
     if (n % 8 != 0 || !aligned16(x) || !aligned16(y)) return BR_ERR_TODO;
-    gelu_fwd_f32_to_f16<<<grid_for(n / 8, kBlock), kBlock, 0, as_stream(stream)>>>((const float4*)x, (half8*)y, n / 8);
+    const int grid = grid_for(n / 8, kBlock);
+    if (y_dtype == BR_F16)
+        gelu_fwd_f32_to_16<__half><<<grid, kBlock, 0, as_stream(stream)>>>((const float4*)x, (uint4*)y, n / 8);
+    else
+        gelu_fwd_f32_to_16<__hip_bfloat16><<<grid, kBlock, 0, as_stream(stream)>>>((const float4*)x, (uint4*)y, n / 8);
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }

@@ -48,7 +48,7 @@ SIGNATURES = {
     "br_hip_cast": (_int, [_vp, _int, _vp, _int, _i64, _vp]),
     "br_hip_add_bcast": (_int, [_vp, _vp, _vp, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), _vp]),
     "br_hip_gelu_fwd": (_int, [_vp, _vp, _int, _i64, _vp]),
-    "br_hip_gelu_fwd_f32_to_f16": (_int, [_vp, _vp, _i64, _vp]),
+    "br_hip_gelu_fwd_f32_to_16": (_int, [_vp, _vp, _int, _i64, _vp]),
     "br_hip_gelu_bwd": (_int, [_vp, _vp, _vp, _int, _i64, _vp]),
     "br_hip_bias_gelu_fwd": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp]),
     "br_hip_bias_gelu_bwd_workspace": (_sz, [_i64, _i64]),

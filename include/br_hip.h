@@ -98,10 +98,10 @@ int br_hip_add_bcast(const void* a, const void* b, void* c, int dtype,
  * dtype is the storage type of x / y / dy / dx (BR_F32 or BR_F16); math is
  * fp32.  dx may alias x. */
 int br_hip_gelu_fwd(const void* x, void* y, int dtype, int64_t n, br_stream_t stream);
-/* The same forward with fp32 x and fp16 y (n % 8 == 0, 16-byte aligned): for an
- * activation that only feeds an fp16 product, which would round an fp32 y the
- * same way. */
-int br_hip_gelu_fwd_f32_to_f16(const float* x, void* y, int64_t n, br_stream_t stream);
+/* The same forward with fp32 x and a 16-bit y (BR_F16 or BR_BF16; n % 8 == 0,
+ * 16-byte aligned): for an activation that only feeds a 16-bit product, which
+ * would round an fp32 y the same way. */
+int br_hip_gelu_fwd_f32_to_16(const float* x, void* y, int y_dtype, int64_t n, br_stream_t stream);
 int br_hip_gelu_bwd(const void* dy, const void* x, void* dx, int dtype, int64_t n,
                     br_stream_t stream);
 

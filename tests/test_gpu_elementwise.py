@@ -153,18 +153,23 @@ def test_colsum_cast_equals_colsum_plus_cast(rows, cols):
     assert_close(host(sums2), x.astype(np.float64).sum(0), RTOL, "colsum")
 
 
-def test_gelu_fwd_f32_to_f16_rounds_the_fp32_result_once():
+def test_gelu_fwd_f32_to_16_rounds_the_fp32_result_once():
+    from gpu_util import BF16
     rng = np.random.default_rng(9)
     n = 8 * 4099
     x = (2.0 * rng.standard_normal(n)).astype(np.float32)
     dx = dev(x)
-    y32, y16 = empty(n), empty(n, torch.float16)
+    y32, y16, yb = empty(n), empty(n, torch.float16), empty(n, torch.bfloat16)
     call("br_hip_gelu_fwd", ptr(dx), ptr(y32), F32, n, stream())
-    call("br_hip_gelu_fwd_f32_to_f16", ptr(dx), ptr(y16), n, stream())
+    call("br_hip_gelu_fwd_f32_to_16", ptr(dx), ptr(y16), F16, n, stream())
+    call("br_hip_gelu_fwd_f32_to_16", ptr(dx), ptr(yb), BF16, n, stream())
     assert np.array_equal(host(y16).view(np.uint16), host(y32).astype(np.float16).view(np.uint16))
+    torch.cuda.synchronize()
+    assert torch.equal(yb, y32.to(torch.bfloat16))
     lib = hip.load()
-    assert lib.br_hip_gelu_fwd_f32_to_f16(ptr(dx), ptr(y16), 12, stream()) == -1      # n % 8 != 0: not this entry's job
-    assert lib.br_hip_gelu_fwd_f32_to_f16(ptr(dx), ptr(y16), 0, stream()) == 0
+    assert lib.br_hip_gelu_fwd_f32_to_16(ptr(dx), ptr(y16), F16, 12, stream()) == -1   # n % 8 != 0: not this entry's job
+    assert lib.br_hip_gelu_fwd_f32_to_16(ptr(dx), ptr(y16), F32, 16, stream()) == -1
+    assert lib.br_hip_gelu_fwd_f32_to_16(ptr(dx), ptr(y16), F16, 0, stream()) == 0
     torch.cuda.synchronize()
 
 
