@@ -618,10 +618,25 @@ template <DataType DT>
 ComputingReturn HIPTensor<DT>::op_softmax_backward(tensor_t self, tensor_t out, tensor_t x_g) {
     if (DT != DataType::Float) return OP_TODO_ERROR;
     if (!dev_f32(out) || out->items() != self->items()) return OP_INPUT_ERROR;
-    if (!dev_f32(x_g) || x_g->items() != self->items()) return OP_OUTPUT_ERROR;
+    if (!dev(x_g) || x_g->items() != self->items()) return OP_OUTPUT_ERROR;
     const int64_t cols = (int64_t)self->shape().vec().back();
-    BR_OP(br_hip_softmax_bwd(static_cast<const float*>(mem_), static_cast<const float*>(out->data()),
-                             static_cast<float*>(x_g->data()), (int64_t)self->items() / cols, cols, stream()));
+    const int64_t rows = (int64_t)self->items() / cols;
+    const float* dy = static_cast<const float*>(mem_);
+    const float* y = static_cast<const float*>(out->data());
+    if (x_g->dtype() != DataType::Float) {
+        // a 16-bit gradient for the score products: written directly when the
+        // kernel can, otherwise fp32 into scratch memory and converted
+        const int rc = br_hip_softmax_bwd_to16(dy, y, x_g->data(), code(x_g), rows, cols, stream());
+        if (rc == BR_ERR_TODO) {
+            float* tmp = static_cast<float*>(ComputingContext::scratch(self->items() * sizeof(float)));
+            BR_OP(br_hip_softmax_bwd(dy, y, tmp, rows, cols, stream()));
+            BR_OP(br_hip_cast(tmp, BR_F32, x_g->data(), code(x_g), (int64_t)self->items(), stream()));
+        } else {
+            BR_OP(rc);
+        }
+        return OP_OK;
+    }
+    BR_OP(br_hip_softmax_bwd(dy, y, static_cast<float*>(x_g->data()), rows, cols, stream()));
     return OP_OK;
 }
 

@@ -34,6 +34,14 @@ struct Tensors {
         NWORD_CREATOR_DEFINE_LR(CLS)                      \
     };
 
+// True when `dst <- src` is the 16-bit device image of the fp32 device tensor
+// `produced` (src is that very tensor).
+bool copy16_of(const tensor_t& dst, const tensor_t& src, const tensor_t& produced) {
+    return dst && src && dst->is_cuda() && (dst->dtype() == DataType::F16 || dst->dtype() == DataType::BF16) &&
+           src->is_cuda() && src->dtype() == DataType::Float && src->data() == produced->data() &&
+           src->items() == produced->items() && dst->items() == src->items();
+}
+
 // ( -- )  wait for everything queued on the compute stream
 BR_WORD(Sync, (void)stack; ComputingContext::sync();)
 
@@ -97,13 +105,16 @@ BR_WORD(Softmax, Tensors<2> a(stack); a[0]->op_softmax(a[0], a[1]);)
 // in place, alibi [1,NH,1,T], xmask [B,1,T,T]) the three passes run as one
 // kernel that applies the same operations in the same order (bit-identical);
 // anything else runs the three operators one after the other.
-BR_WORD(AddAddSoftmax,
-    Tensors<8> a(stack);
+// `copy_dst` / `copy_src` (both null, or the operands of an `op.copy` that
+// follows): when the copy is a 16-bit image of the softmax output, the fused
+// kernel writes it too.
+void add_add_softmax(Tensors<8>& a, const tensor_t& copy_dst, const tensor_t& copy_src) {
     auto same = [](const tensor_t& x, const tensor_t& y) { return x->data() == y->data() && x->items() == y->items(); };
     auto f32dev = [](const tensor_t& x) { return x->is_cuda() && x->dtype() == DataType::Float; };
     bool fast = f32dev(a[0]) && f32dev(a[1]) && f32dev(a[4]) && f32dev(a[7]) && a[0]->shape().dim() == 4 &&
                 a[1]->shape().dim() == 4 && a[4]->shape().dim() == 4 && same(a[0], a[2]) && same(a[0], a[3]) &&
                 same(a[0], a[5]) && same(a[0], a[6]) && a[7]->items() == a[0]->items();
+    bool copied = false;
     if (fast) {
         const auto& xs = a[0]->shape();
         const auto& as = a[1]->shape();
@@ -111,16 +122,70 @@ BR_WORD(AddAddSoftmax,
         fast = as[0] == 1 && as[1] == xs[1] && as[2] == 1 && as[3] == xs[3] && ms[0] == xs[0] && ms[1] == 1 &&
                ms[2] == xs[2] && ms[3] == xs[3];
         if (fast) {
-            BR_HIP_CHECK(br_hip_alibi_masked_softmax_fwd(
-                static_cast<const float*>(a[0]->data()), static_cast<const float*>(a[1]->data()),
-                static_cast<const float*>(a[4]->data()), static_cast<float*>(a[7]->data()), (int64_t)xs[0],
-                (int64_t)xs[1], (int64_t)xs[2], (int64_t)xs[3], ComputingContext::stream));
+            const float* x = static_cast<const float*>(a[0]->data());
+            const float* alibi = static_cast<const float*>(a[1]->data());
+            const float* mask = static_cast<const float*>(a[4]->data());
+            float* out = static_cast<float*>(a[7]->data());
+            if (copy_dst && copy16_of(copy_dst, copy_src, a[7])) {
+                const int rc = br_hip_alibi_masked_softmax_fwd_copy16(
+                    x, alibi, mask, out, copy_dst->data(), (int)copy_dst->dtype(), (int64_t)xs[0], (int64_t)xs[1],
+                    (int64_t)xs[2], (int64_t)xs[3], ComputingContext::stream);
+                if (rc != BR_ERR_TODO) {
+                    BR_HIP_CHECK(rc);
+                    copied = true;
+                }
+            }
+            if (!copied)
+                BR_HIP_CHECK(br_hip_alibi_masked_softmax_fwd(x, alibi, mask, out, (int64_t)xs[0], (int64_t)xs[1],
+                                                             (int64_t)xs[2], (int64_t)xs[3],
+                                                             ComputingContext::stream));
         }
     }
     if (!fast) {
         a[0]->op_add(a[0], a[1], a[2]);
         a[3]->op_add(a[3], a[4], a[5]);
         a[6]->op_softmax(a[6], a[7]);
+    }
+    if (copy_dst && !copied) copy_dst->op_copy(copy_dst, copy_src);
+}
+BR_WORD(AddAddSoftmax, Tensors<8> a(stack); add_add_softmax(a, nullptr, nullptr);)
+// ( x a x  x m x  x y  dst src -- )  the same followed by `op.copy`
+BR_WORD(AddAddSoftmaxCopy,
+    Tensors<2> c(stack);
+    Tensors<8> a(stack);
+    add_add_softmax(a, c[0], c[1]);
+)
+// ( x mean var scale bias y eps  dst src -- )  `op.layernorm` followed by
+// `op.copy`: when the copy is a 16-bit image of y the forward kernel writes
+// both; anything else runs the two operators one after the other.
+BR_WORD(LayernormCopy,
+    Tensors<2> c(stack);
+    const float eps = (float)stack.pop_number();
+    Tensors<6> a(stack);
+    auto f32dev = [](const tensor_t& x) { return x->is_cuda() && x->dtype() == DataType::Float; };
+    bool done = false;
+    bool fast = copy16_of(c[0], c[1], a[5]) && a[0]->shape().dim() == 3;
+    for (size_t i = 0; i < 6; i++) fast = fast && f32dev(a[i]);
+    if (fast) {
+        const int64_t rows = (int64_t)(a[0]->shape()[0] * a[0]->shape()[1]);
+        const int64_t cols = (int64_t)a[0]->shape()[2];
+        fast = (int64_t)a[1]->items() >= rows && (int64_t)a[2]->items() >= rows && (int64_t)a[3]->items() == cols &&
+               (int64_t)a[4]->items() == cols && a[5]->items() == a[0]->items();
+        if (fast) {
+            const int rc = br_hip_layernorm_fwd_copy16(
+                static_cast<const float*>(a[0]->data()), static_cast<const float*>(a[3]->data()),
+                static_cast<const float*>(a[4]->data()), static_cast<float*>(a[5]->data()), c[0]->data(),
+                (int)c[0]->dtype(), static_cast<float*>(a[1]->data()), static_cast<float*>(a[2]->data()), rows, cols,
+                eps, ComputingContext::stream);
+            if (rc != BR_ERR_TODO) {
+                BR_HIP_CHECK(rc);
+                done = true;
+            }
+        }
+    }
+    if (!done) {
+        a[0]->op_layernorm(a[0], a[1], a[2], a[3], a[4], a[5], eps);
+        c[0]->op_copy(c[0], c[1]);
     }
 )
 // ( p v out -- )
@@ -188,6 +253,8 @@ void load_nn_words(Enviroment& env) {
         {"op.querykey", QueryKey::creator},
         {"op.softmax", Softmax::creator},
         {"op.add_add_softmax", AddAddSoftmax::creator},
+        {"op.add_add_softmax_copy", AddAddSoftmaxCopy::creator},
+        {"op.layernorm_copy", LayernormCopy::creator},
         {"op.attn", Attn::creator},
         {"op.gelu", Gelu::creator},
         {"op.last_logits", LastLogits::creator},
@@ -201,7 +268,10 @@ void load_nn_words(Enviroment& env) {
         {"op.qk_backward", QueryKeyBackward::creator},
     };
     for (const auto& e : table) env.insert_native_word(e.name, e.creator);
+    // longer patterns first: a pass only sees what earlier passes left unfused
+    env.insert_fusion({"op.add", "op.add", "op.softmax", "op.copy"}, "op.add_add_softmax_copy");
     env.insert_fusion({"op.add", "op.add", "op.softmax"}, "op.add_add_softmax");
+    env.insert_fusion({"op.layernorm", "op.copy"}, "op.layernorm_copy");
 }
 
 }  // namespace br

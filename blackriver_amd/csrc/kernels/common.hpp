@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
@@ -87,6 +88,38 @@ __device__ __forceinline__ half8 pack8(const float (&f)[8]) {
 #pragma unroll
     for (int i = 0; i < 4; i++) h.v[i] = __floats2half2_rn(f[2 * i], f[2 * i + 1]);
     return h;
+}
+
+// Optional second output of an fp32-producing kernel: the same values rounded
+// to fp16 / bf16, for consumers that are 16-bit matrix products.  `base` is a
+// dense array with the fp32 output's indexing; null = no copy.
+struct Copy16 {
+    void* base;
+    int bf16;
+};
+// Stores v (4 consecutive fp32 results, already final) at 4-element index idx4.
+// The barrier keeps the fp32 rounding: without it the compiler may fold the
+// producing multiply-add into the conversion, and the copy would differ from
+// the rounded fp32 output in the last bit.
+__device__ __forceinline__ void store4_as16(const Copy16& c, int64_t idx4, float4& v) {
+    asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w));
+    if (!c.base) return;
+    unsigned lo, hi;
+    if (c.bf16) {
+        lo = (unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(v.x)) |
+             ((unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(v.y)) << 16);
+        hi = (unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(v.z)) |
+             ((unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(v.w)) << 16);
+    } else {
+        lo = (unsigned)__builtin_bit_cast(unsigned short, __float2half_rn(v.x)) |
+             ((unsigned)__builtin_bit_cast(unsigned short, __float2half_rn(v.y)) << 16);
+        hi = (unsigned)__builtin_bit_cast(unsigned short, __float2half_rn(v.z)) |
+             ((unsigned)__builtin_bit_cast(unsigned short, __float2half_rn(v.w)) << 16);
+    }
+    reinterpret_cast<uint2*>(c.base)[idx4] = make_uint2(lo, hi);
+}
+inline bool copy16_ok(const void* y16, int dtype) {
+    return y16 && (dtype == BR_F16 || dtype == BR_BF16) && (reinterpret_cast<uintptr_t>(y16) & 7u) == 0;
 }
 
 // Grid size for a grid-stride elementwise kernel: enough workgroups to keep

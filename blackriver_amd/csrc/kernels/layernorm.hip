@@ -32,7 +32,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_regs(const float* __restrict__ 
                                                        const float* __restrict__ beta,
                                                        float* __restrict__ y, float* __restrict__ mean_out,
                                                        float* __restrict__ var_out, int cols4, float eps,
-                                                       float inv_cols) {
+                                                       float inv_cols, Copy16 y16) {
     __shared__ float lds[2][kWaves];
     const int64_t row = blockIdx.x;
     const float4* xr = reinterpret_cast<const float4*>(x) + row * cols4;
@@ -76,6 +76,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_regs(const float* __restrict__ 
             o.y = (v[i].y - mean) * rstd * g.y + b.y;
             o.z = (v[i].z - mean) * rstd * g.z + b.z;
             o.w = (v[i].w - mean) * rstd * g.w + b.w;
+            store4_as16(y16, row * cols4 + idx, o);
             yr[idx] = o;
         }
     }
@@ -331,6 +332,31 @@ bool regs_path_ok(int64_t cols, const void* a, const void* b, const void* c, con
 
 }  // namespace
 
+namespace {
+int layernorm_fwd_launch(const float* x, const float* gamma, const float* beta, float* y, Copy16 y16, float* mean,
+                         float* var, int64_t rows, int64_t cols, float eps, hipStream_t st) {
+    const unsigned grid = (unsigned)rows;
+    if (regs_path_ok(cols, x, gamma, beta, y, y)) {
+        const int cols4 = (int)(cols / 4);
+        const float inv = 1.0f / (float)cols;
+        const int vpt = (cols4 + kBlock - 1) / kBlock;
+        if (vpt <= 1)
+            ln_fwd_regs<1><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv, y16);
+        else if (vpt <= 2)
+            ln_fwd_regs<2><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv, y16);
+        else if (vpt <= 4)
+            ln_fwd_regs<4><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv, y16);
+        else
+            ln_fwd_regs<8><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv, y16);
+    } else {
+        if (y16.base) return BR_ERR_TODO;  // the copy is only produced by the register path
+        ln_fwd_generic<<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols, eps);
+    }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+}  // namespace
+
 extern "C" {
 
 int br_hip_layernorm_fwd(const float* x, const float* gamma, const float* beta, float* y, float* mean,
@@ -339,25 +365,19 @@ int br_hip_layernorm_fwd(const float* x, const float* gamma, const float* beta, 
     if (rows == 0) return BR_OK;
     if (!x || !gamma || !beta) return BR_ERR_INPUT;
     if (!y) return BR_ERR_OUTPUT;
-    hipStream_t st = as_stream(stream);
-    const unsigned grid = (unsigned)rows;
-    if (regs_path_ok(cols, x, gamma, beta, y, y)) {
-        const int cols4 = (int)(cols / 4);
-        const float inv = 1.0f / (float)cols;
-        const int vpt = (cols4 + kBlock - 1) / kBlock;
-        if (vpt <= 1)
-            ln_fwd_regs<1><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
-        else if (vpt <= 2)
-            ln_fwd_regs<2><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
-        else if (vpt <= 4)
-            ln_fwd_regs<4><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
-        else
-            ln_fwd_regs<8><<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols4, eps, inv);
-    } else {
-        ln_fwd_generic<<<grid, kBlock, 0, st>>>(x, gamma, beta, y, mean, var, cols, eps);
-    }
-    BR_HIP_LAUNCH_CHECK();
-    return BR_OK;
+    return layernorm_fwd_launch(x, gamma, beta, y, Copy16{nullptr, 0}, mean, var, rows, cols, eps, as_stream(stream));
+}
+
+int br_hip_layernorm_fwd_copy16(const float* x, const float* gamma, const float* beta, float* y, void* y16,
+                                int y16_dtype, float* mean, float* var, int64_t rows, int64_t cols, float eps,
+                                br_stream_t stream) {
+    if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!x || !gamma || !beta) return BR_ERR_INPUT;
+    if (!y || !y16) return BR_ERR_OUTPUT;
+    if (!copy16_ok(y16, y16_dtype) || !regs_path_ok(cols, x, gamma, beta, y, y)) return BR_ERR_TODO;
+    return layernorm_fwd_launch(x, gamma, beta, y, Copy16{y16, y16_dtype == BR_BF16}, mean, var, rows, cols, eps,
+                                as_stream(stream));
 }
 
 size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols) {

@@ -35,7 +35,7 @@ __device__ __forceinline__ float exp_sub(float x, float m) { return __expf(x - m
 // VPL = float4 vectors per lane; cols = 4 * cols4 <= 256 * VPL.
 template <int VPL, int MODE>
 __global__ __launch_bounds__(kBlock) void softmax_fwd_wave(const float* __restrict__ x, float* __restrict__ y,
-                                                            int64_t rows, int cols4, RowBias rb) {
+                                                            int64_t rows, int cols4, RowBias rb, Copy16 y16) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -106,13 +106,18 @@ __global__ __launch_bounds__(kBlock) void softmax_fwd_wave(const float* __restri
 #pragma unroll
     for (int i = 0; i < VPL; i++) {
         const int idx = lane + i * kWave;
-        if (idx < cols4) yr[idx] = make_float4(v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+        if (idx < cols4) {
+            float4 o = make_float4(v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
+            store4_as16(y16, row * cols4 + idx, o);
+            yr[idx] = o;
+        }
     }
 }
 
 template <int VPL>
 __global__ __launch_bounds__(kBlock) void softmax_bwd_wave(const float* __restrict__ dy, const float* __restrict__ y,
-                                                            float* __restrict__ dx, int64_t rows, int cols4) {
+                                                            float* __restrict__ dx, int64_t rows, int cols4,
+                                                            Copy16 dx16) {
     const int lane = threadIdx.x & 63;
     const int64_t row = (int64_t)blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
     if (row >= rows) return;
@@ -129,13 +134,16 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_wave(const float* __restri
         dot += (g[i].x * p[i].x + g[i].y * p[i].y) + (g[i].z * p[i].z + g[i].w * p[i].w);
     }
     dot = wave_sum(dot);
-    float4* dr = reinterpret_cast<float4*>(dx) + row * cols4;
+    float4* dr = dx ? reinterpret_cast<float4*>(dx) + row * cols4 : nullptr;
 #pragma unroll
     for (int i = 0; i < VPL; i++) {
         const int idx = lane + i * kWave;
-        if (idx < cols4)
-            dr[idx] = make_float4(p[i].x * (g[i].x - dot), p[i].y * (g[i].y - dot), p[i].z * (g[i].z - dot),
-                                  p[i].w * (g[i].w - dot));
+        if (idx < cols4) {
+            float4 o = make_float4(p[i].x * (g[i].x - dot), p[i].y * (g[i].y - dot), p[i].z * (g[i].z - dot),
+                                   p[i].w * (g[i].w - dot));
+            store4_as16(dx16, row * cols4 + idx, o);
+            if (dx) dr[idx] = o;  // dx == nullptr: only the 16-bit gradient is wanted
+        }
     }
 }
 
@@ -188,7 +196,8 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_generic(const float* dy, c
 }
 
 template <int MODE>
-int launch_softmax_fwd(const float* x, float* y, int64_t rows, int64_t cols, const RowBias& rb, hipStream_t st) {
+int launch_softmax_fwd(const float* x, float* y, int64_t rows, int64_t cols, const RowBias& rb, hipStream_t st,
+                       Copy16 y16 = Copy16{nullptr, 0}) {
     bool vec = cols % 4 == 0 && cols <= 256 * 16 && aligned16(x) && aligned16(y);
     if (MODE == kTables)
         vec = vec && (!rb.alibi || aligned16(rb.alibi)) && (!rb.xmask || aligned16(rb.xmask));
@@ -197,18 +206,40 @@ int launch_softmax_fwd(const float* x, float* y, int64_t rows, int64_t cols, con
         const unsigned grid = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
         const int vpl = (cols4 + kWave - 1) / kWave;
         if (vpl <= 1)
-            softmax_fwd_wave<1, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb);
+            softmax_fwd_wave<1, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb, y16);
         else if (vpl <= 2)
-            softmax_fwd_wave<2, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb);
+            softmax_fwd_wave<2, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb, y16);
         else if (vpl <= 4)
-            softmax_fwd_wave<4, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb);
+            softmax_fwd_wave<4, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb, y16);
         else if (vpl <= 8)
-            softmax_fwd_wave<8, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb);
+            softmax_fwd_wave<8, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb, y16);
         else
-            softmax_fwd_wave<16, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb);
+            softmax_fwd_wave<16, MODE><<<grid, kBlock, 0, st>>>(x, y, rows, cols4, rb, y16);
     } else {
+        if (y16.base) return BR_ERR_TODO;  // the copy is only produced by the one-wave-per-row path
         softmax_fwd_generic<MODE><<<(unsigned)rows, kBlock, 0, st>>>(x, y, cols, rb);
     }
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+bool softmax_bwd_wave_ok(int64_t cols, const void* dy, const void* y, const void* dx) {
+    return cols % 4 == 0 && cols <= 256 * 8 && aligned16(dy) && aligned16(y) && aligned16(dx);
+}
+
+int launch_softmax_bwd_wave(const float* dy, const float* y, float* dx, Copy16 dx16, int64_t rows, int64_t cols,
+                            hipStream_t st) {
+    const int cols4 = (int)(cols / 4);
+    const unsigned grid = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
+    const int vpl = (cols4 + kWave - 1) / kWave;
+    if (vpl <= 1)
+        softmax_bwd_wave<1><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4, dx16);
+    else if (vpl <= 2)
+        softmax_bwd_wave<2><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4, dx16);
+    else if (vpl <= 4)
+        softmax_bwd_wave<4><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4, dx16);
+    else
+        softmax_bwd_wave<8><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4, dx16);
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }
@@ -385,23 +416,20 @@ int br_hip_softmax_bwd(const float* dy, const float* y, float* dx, int64_t rows,
     if (!dy || !y) return BR_ERR_INPUT;
     if (!dx) return BR_ERR_OUTPUT;
     hipStream_t st = as_stream(stream);
-    if (cols % 4 == 0 && cols <= 256 * 8 && aligned16(dy) && aligned16(y) && aligned16(dx)) {
-        const int cols4 = (int)(cols / 4);
-        const unsigned grid = (unsigned)((rows + kRowsPerBlock - 1) / kRowsPerBlock);
-        const int vpl = (cols4 + kWave - 1) / kWave;
-        if (vpl <= 1)
-            softmax_bwd_wave<1><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4);
-        else if (vpl <= 2)
-            softmax_bwd_wave<2><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4);
-        else if (vpl <= 4)
-            softmax_bwd_wave<4><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4);
-        else
-            softmax_bwd_wave<8><<<grid, kBlock, 0, st>>>(dy, y, dx, rows, cols4);
-    } else {
-        softmax_bwd_generic<<<(unsigned)rows, kBlock, 0, st>>>(dy, y, dx, cols);
-    }
+    if (softmax_bwd_wave_ok(cols, dy, y, dx)) return launch_softmax_bwd_wave(dy, y, dx, Copy16{nullptr, 0}, rows, cols, st);
+    softmax_bwd_generic<<<(unsigned)rows, kBlock, 0, st>>>(dy, y, dx, cols);
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
+}
+
+int br_hip_softmax_bwd_to16(const float* dy, const float* y, void* dx16, int dx16_dtype, int64_t rows, int64_t cols,
+                            br_stream_t stream) {
+    if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!dy || !y) return BR_ERR_INPUT;
+    if (!dx16 || dx16 == (const void*)dy || dx16 == (const void*)y) return BR_ERR_OUTPUT;
+    if (!copy16_ok(dx16, dx16_dtype) || !softmax_bwd_wave_ok(cols, dy, y, dy)) return BR_ERR_TODO;
+    return launch_softmax_bwd_wave(dy, y, nullptr, Copy16{dx16, dx16_dtype == BR_BF16}, rows, cols, as_stream(stream));
 }
 
 int br_hip_alibi_masked_softmax_fwd(const float* s, const float* alibi, const float* xmask, float* p,
@@ -415,6 +443,21 @@ int br_hip_alibi_masked_softmax_fwd(const float* s, const float* alibi, const fl
     if (!p) return BR_ERR_OUTPUT;
     RowBias rb = {alibi, xmask, nullptr, nullptr, (int)heads, (int)tq};
     return launch_softmax_fwd<kTables>(s, p, rows, tk, rb, as_stream(stream));
+}
+
+int br_hip_alibi_masked_softmax_fwd_copy16(const float* s, const float* alibi, const float* xmask, float* p, void* p16,
+                                           int p16_dtype, int64_t batch, int64_t heads, int64_t tq, int64_t tk,
+                                           br_stream_t stream) {
+    if (batch < 0 || heads <= 0 || tq <= 0 || tk <= 0 || heads > 0x7fffffff || tq > 0x7fffffff)
+        return BR_ERR_ATTR;
+    const int64_t rows = batch * heads * tq;
+    if (rows > 0x7fffffff) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!s) return BR_ERR_INPUT;
+    if (!p || !p16) return BR_ERR_OUTPUT;
+    if (!copy16_ok(p16, p16_dtype)) return BR_ERR_TODO;
+    RowBias rb = {alibi, xmask, nullptr, nullptr, (int)heads, (int)tq};
+    return launch_softmax_fwd<kTables>(s, p, rows, tk, rb, as_stream(stream), Copy16{p16, p16_dtype == BR_BF16});
 }
 
 int br_hip_alibi_causal_softmax_fwd(const float* s, const double* slopes, const int32_t* valid, float* p,

@@ -58,10 +58,13 @@ SIGNATURES = {
     "br_hip_colsum_cast": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp, _sz, _vp]),
     "br_hip_colsum": (_int, [_vp, _int, _vp, _i64, _i64, _vp, _sz, _vp]),
     "br_hip_layernorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
+    "br_hip_layernorm_fwd_copy16": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _f32, _vp]),
     "br_hip_layernorm_bwd_workspace": (_sz, [_i64, _i64]),
     "br_hip_layernorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp, _sz, _vp]),
     "br_hip_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "br_hip_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
+    "br_hip_softmax_bwd_to16": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp]),
+    "br_hip_alibi_masked_softmax_fwd_copy16": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "br_hip_alibi_masked_softmax_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "br_hip_alibi_causal_softmax_fwd": (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp]),
     "br_hip_logsoftmax_nll_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),

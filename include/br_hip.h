@@ -144,6 +144,16 @@ int br_hip_layernorm_fwd(const float* x, const float* gamma, const float* beta, 
                          float* mean, float* var, int64_t rows, int64_t cols, float eps,
                          br_stream_t stream);
 
+/* The same forward, which also writes y rounded to nearest as fp16 / bf16
+ * (y16_dtype = BR_F16 / BR_BF16) into y16: the `op.layernorm` + `op.copy`
+ * pair of a script whose next consumer is a 16-bit matrix product
+ * (cuda_tensor.cpp:236-255 followed by op_copy, :128-144), in one pass over x.  y16 holds
+ * exactly what a cast of y would.  BR_ERR_TODO when the shape or alignment
+ * needs the general kernel: the caller then runs the two steps separately. */
+int br_hip_layernorm_fwd_copy16(const float* x, const float* gamma, const float* beta, float* y,
+                                void* y16, int y16_dtype, float* mean, float* var, int64_t rows,
+                                int64_t cols, float eps, br_stream_t stream);
+
 /* kernels::launch_ln_bw_float, kernels/normalize_kernels.cu:361-383
  * (declared kernels/kernels.h:28) with means == nullptr, called at cuda_tensor.cpp:699-727.  y is the forward
  * OUTPUT, var what the forward stored; dgamma / dbeta are overwritten. */
@@ -161,6 +171,14 @@ int br_hip_softmax_fwd(const float* x, float* y, int64_t rows, int64_t cols,
 int br_hip_softmax_bwd(const float* dy, const float* y, float* dx, int64_t rows, int64_t cols,
                        br_stream_t stream);
 
+/* cudnnSoftmaxBackward at cuda_tensor.cpp:890-918 with the gradient stored
+ * only as fp16 / bf16 (round to nearest of the fp32 value br_hip_softmax_bwd
+ * stores), for a consumer that is a 16-bit matrix product
+ * (op_qk_backward, cuda_tensor.cpp:1006).  dx16 must not alias the inputs.
+ * BR_ERR_TODO when the rows do not fit the one-wave-per-row kernel. */
+int br_hip_softmax_bwd_to16(const float* dy, const float* y, void* dx16, int dx16_dtype,
+                            int64_t rows, int64_t cols, br_stream_t stream);
+
 /* The three-word sequence of bloomz-7b/train.words:158-162 in one pass:
  * p = softmax((s + alibi[h,:]) + xmask[b,q,:]) over the last dimension of
  * s[batch, heads, tq, tk], with alibi[heads, tk] and xmask[batch, tq, tk]
@@ -169,6 +187,15 @@ int br_hip_softmax_bwd(const float* dy, const float* y, float* dx, int64_t rows,
 int br_hip_alibi_masked_softmax_fwd(const float* s, const float* alibi, const float* xmask,
                                     float* p, int64_t batch, int64_t heads, int64_t tq,
                                     int64_t tk, br_stream_t stream);
+
+/* br_hip_alibi_masked_softmax_fwd, which also writes p rounded to nearest as
+ * fp16 / bf16 into p16 (what a cast of p would hold), so that the attention
+ * product can read the 16-bit probabilities while the backward keeps the fp32
+ * ones.  BR_ERR_TODO when the rows do not fit the one-wave-per-row kernel. */
+int br_hip_alibi_masked_softmax_fwd_copy16(const float* s, const float* alibi,
+                                           const float* xmask, float* p, void* p16,
+                                           int p16_dtype, int64_t batch, int64_t heads,
+                                           int64_t tq, int64_t tk, br_stream_t stream);
 
 /* The same, with the ALiBi bias and the causal / padding mask of
  * blackriver/train_bloom.cpp:58-90 computed in the kernel from the device

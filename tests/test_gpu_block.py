@@ -128,10 +128,13 @@ def test_operand_buffer_words_give_the_same_bits(runtime, mode, hidden, heads, b
     env.write("xinput", x)
     env.execute("block_step_mixed op.sync")
     for n in names:
-        assert np.array_equal(env.read(n), plain[n]), n
-    # the buffers hold what the fp32 tensors round to
+        if n != "xll":
+            assert np.array_equal(env.read(n), plain[n]), n
+    # the buffers hold what the fp32 tensors round to; the score gradient, which
+    # the fp32-arena words leave in xll, exists only as its 16-bit image here
     if mode == "f16":
         assert np.array_equal(env.read("xattn_in.h"), env.read("xattn_in").astype(np.float16).astype(np.float32))
+        assert np.array_equal(env.read("xll.h"), plain["xll"].astype(np.float16).astype(np.float32))
     env.close()
 
 

@@ -7,7 +7,7 @@ import torch
 
 import oracle as orc
 from conftest import assert_close
-from gpu_util import call, dev, empty, host, ptr, stream, workspace
+from gpu_util import BF16, F16, F32, call, dev, empty, host, ptr, stream, workspace
 from blackriver_amd import hip
 
 pytestmark = pytest.mark.gpu
@@ -98,4 +98,41 @@ def test_layernorm_rejects_bad_arguments():
     assert lib.br_hip_layernorm_fwd(ptr(t), ptr(t), ptr(t), ptr(t), None, None, 1, 0, 1e-5, stream()) == -4
     assert lib.br_hip_layernorm_bwd(ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 1, 16, 1e-5,
                                     None, 0, stream()) == -4
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype,tdtype", [(F16, torch.float16), (BF16, torch.bfloat16)])
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (3, 64), (5, 8192), (9, 1000)])
+def test_layernorm_fwd_with_16_bit_copy(rows, cols, dtype, tdtype):
+    """The forward that also writes a 16-bit image of y: y, mean and var are
+    bit for bit the plain forward's, and the image is bit for bit the cast of
+    y (so scripts may use either form)."""
+    print("case rows=%d cols=%d dtype=%d" % (rows, cols, dtype), flush=True)
+    x, g, b, _ = make(rows, cols, seed=3)
+    eps = 1e-5
+    y_plain, mean_plain, var_plain = run_fwd(x, g, b, eps)
+    y, mean, var = empty((rows, cols)), empty(rows), empty(rows)
+    y16 = empty((rows, cols), tdtype)
+    call("br_hip_layernorm_fwd_copy16", ptr(dev(x)), ptr(dev(g)), ptr(dev(b)), ptr(y), ptr(y16), dtype, ptr(mean),
+         ptr(var), rows, cols, eps, stream())
+    assert np.array_equal(host(y), y_plain)
+    assert np.array_equal(host(mean), mean_plain) and np.array_equal(host(var), var_plain)
+    cast = empty((rows, cols), tdtype)
+    call("br_hip_cast", ptr(y), F32, ptr(cast), dtype, rows * cols, stream())
+    assert torch.equal(y16.view(torch.int16), cast.view(torch.int16))
+    assert torch.equal(y16, y.to(tdtype))   # round to nearest even of the fp32 output
+
+
+def test_layernorm_fwd_with_16_bit_copy_declines_what_the_row_kernel_cannot_do():
+    lib = hip.load()
+    rows, cols = 4, 1001   # not a multiple of 4: general kernel, no copy
+    t = empty(rows * cols)
+    g = empty(cols)
+    h = empty(rows * cols, torch.float16)
+    assert lib.br_hip_layernorm_fwd_copy16(ptr(t), ptr(g), ptr(g), ptr(t), ptr(h), F16, None, None, rows, cols, 1e-5,
+                                           stream()) == -1
+    assert lib.br_hip_layernorm_fwd_copy16(ptr(t), ptr(g), ptr(g), ptr(t), ptr(h), F32, None, None, rows, 1000, 1e-5,
+                                           stream()) == -1
+    assert lib.br_hip_layernorm_fwd_copy16(ptr(t), ptr(g), ptr(g), ptr(t), None, F16, None, None, rows, 1000, 1e-5,
+                                           stream()) == -3
     torch.cuda.synchronize()

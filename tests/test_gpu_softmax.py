@@ -9,7 +9,7 @@ import torch
 
 import oracle as orc
 from conftest import assert_close
-from gpu_util import F16, F32, assert_close_f16, call, dev, empty, host, ptr, stream
+from gpu_util import BF16, F16, F32, assert_close_f16, call, dev, empty, host, ptr, stream
 from blackriver_amd import hip
 
 pytestmark = pytest.mark.gpu
@@ -218,5 +218,116 @@ def test_fused_add_add_softmax_word_is_bit_identical_to_the_three_words(runtime)
         env.execute("'p' @ op.zero 'q' @ op.zero")
         env.execute("  ".join(other))
         assert np.array_equal(env.read("p"), expect_p) and np.array_equal(env.read("q"), expect_q)
+    finally:
+        env.close()
+
+
+@pytest.mark.parametrize("dtype,tdtype", [(F16, torch.float16), (BF16, torch.bfloat16)])
+@pytest.mark.parametrize("b,h,t", [(2, 32, 512), (1, 3, 36), (1, 2, 2048)])
+def test_softmax_16_bit_outputs_are_the_cast_of_the_fp32_outputs(b, h, t, dtype, tdtype):
+    """The fused score softmax with a 16-bit image of p, and the softmax
+    backward that stores only a 16-bit gradient, against the plain kernels
+    followed by a cast: identical bits."""
+    print("case b=%d h=%d t=%d dtype=%d" % (b, h, t, dtype), flush=True)
+    rng = np.random.default_rng(21)
+    s = rng.standard_normal((b, h, t, t)).astype(np.float32)
+    alibi = orc.alibi(h, t)
+    mask = np.ones((b, t), np.int32)
+    mask[0, t - 5:] = 0
+    xmask = orc.xmask(mask)
+    ds, da, dm = dev(s), dev(alibi), dev(xmask)
+    p_plain = empty(s.shape)
+    call("br_hip_alibi_masked_softmax_fwd", ptr(ds), ptr(da), ptr(dm), ptr(p_plain), b, h, t, t, stream())
+    p, p16 = empty(s.shape), empty(s.shape, tdtype)
+    call("br_hip_alibi_masked_softmax_fwd_copy16", ptr(ds), ptr(da), ptr(dm), ptr(p), ptr(p16), dtype, b, h, t, t,
+         stream())
+    assert torch.equal(p, p_plain)
+    assert torch.equal(p16, p_plain.to(tdtype))
+    # in place on the scores, as the scripts run it
+    call("br_hip_alibi_masked_softmax_fwd_copy16", ptr(ds), ptr(da), ptr(dm), ptr(ds), ptr(p16), dtype, b, h, t, t,
+         stream())
+    assert torch.equal(ds, p_plain) and torch.equal(p16, p_plain.to(tdtype))
+
+    dp = dev(rng.standard_normal(s.shape).astype(np.float32))
+    g_plain = empty(s.shape)
+    call("br_hip_softmax_bwd", ptr(dp), ptr(p_plain), ptr(g_plain), b * h * t, t, stream())
+    g16 = empty(s.shape, tdtype)
+    call("br_hip_softmax_bwd_to16", ptr(dp), ptr(p_plain), ptr(g16), dtype, b * h * t, t, stream())
+    assert torch.equal(g16, g_plain.to(tdtype))
+    torch.cuda.synchronize()
+
+
+def test_softmax_16_bit_outputs_decline_rows_the_wave_kernel_cannot_hold():
+    lib = hip.load()
+    rows, cols = 3, 1001
+    t = empty(rows * cols)
+    h16 = empty(rows * cols, torch.float16)
+    assert lib.br_hip_softmax_bwd_to16(ptr(t), ptr(t), ptr(h16), F16, rows, cols, stream()) == -1
+    assert lib.br_hip_softmax_bwd_to16(ptr(t), ptr(t), ptr(h16), F32, rows, 1000, stream()) == -1
+    assert lib.br_hip_alibi_masked_softmax_fwd_copy16(ptr(t), None, None, ptr(t), ptr(h16), F16, 1, 1, rows, cols,
+                                                      stream()) == -1
+    assert lib.br_hip_alibi_masked_softmax_fwd_copy16(ptr(t), None, None, ptr(t), None, F16, 1, 1, rows, 1000,
+                                                      stream()) == -3
+    torch.cuda.synchronize()
+
+
+def test_fused_words_with_a_16_bit_copy_match_the_separate_words(runtime):
+    """`op.layernorm op.copy` and `op.add op.add op.softmax op.copy` are fused
+    when the copy is the 16-bit image of the output; run fused (one program)
+    and separately (one program per word) they must leave identical tensors.
+    A copy of something else leaves the sequence to the fallback.  A 16-bit
+    `op.softmax_backward` output equals the cast of the fp32 one."""
+    from blackriver_amd import host
+    rng = np.random.default_rng(5)
+    b, h, t, hid = 2, 4, 96, 256
+    env = host.Env(1)
+    try:
+        env.execute("%d %d %d 3 'cuda' 'float' op.create 'x' !  %d %d %d 3 'cuda' 'float' op.create 'y' !"
+                    % (b, t, hid, b, t, hid))
+        env.execute("%d %d %d 3 'cuda' 'f16' op.create 'y.h' !  %d %d %d 3 'cuda' 'f16' op.create 'z.h' !"
+                    % (b, t, hid, b, t, hid))
+        env.execute("%d 1 'cuda' 'float' op.create 'mean' !  %d 1 'cuda' 'float' op.create 'var' !" % (b * t, b * t))
+        env.execute("%d 1 'cuda' 'float' op.create 'g' !  %d 1 'cuda' 'float' op.create 'bb' !" % (hid, hid))
+        env.write("x", rng.standard_normal((b, t, hid)).astype(np.float32))
+        env.write("g", (1 + 0.1 * rng.standard_normal(hid)).astype(np.float32))
+        env.write("bb", (0.1 * rng.standard_normal(hid)).astype(np.float32))
+        ln = "'x' @ 'mean' @ 'var' @ 'g' @ 'bb' @ 'y' @ 1e-5 op.layernorm"
+        for cp in ("'y.h' @ 'y' @ op.copy", "'z.h' @ 'x' @ op.copy"):
+            dst = cp.split("'")[1]
+            env.execute(ln)
+            env.execute(cp)
+            y_sep, c_sep = env.read("y"), env.read(dst)
+            env.execute("'y' @ op.zero '%s' @ op.zero" % dst)
+            env.execute(ln + "  " + cp)
+            assert np.array_equal(env.read("y"), y_sep)
+            assert np.array_equal(env.read(dst).view(np.int16), c_sep.view(np.int16))
+
+        env.execute("%d %d %d %d 4 'cuda' 'float' op.create 's' !  %d %d %d %d 4 'cuda' 'f16' op.create 's.h' !"
+                    % (b, h, t, t, b, h, t, t))
+        env.execute("1 %d 1 %d 4 'cuda' 'float' op.create 'a' !  %d 1 %d %d 4 'cuda' 'float' op.create 'm' !"
+                    % (h, t, b, t, t))
+        s = rng.standard_normal((b, h, t, t)).astype(np.float32)
+        env.write("a", rng.standard_normal((1, h, 1, t)).astype(np.float32))
+        env.write("m", np.where(rng.random((b, 1, t, t)) < 0.3, -3.4028234663852886e38, 0.0).astype(np.float32))
+        words = ["'s' @ 'a' @ 's' @ op.add", "'s' @ 'm' @ 's' @ op.add", "'s' @ 's' @ op.softmax",
+                 "'s.h' @ 's' @ op.copy"]
+        env.write("s", s)
+        for w in words:
+            env.execute(w)
+        p_sep, h_sep = env.read("s"), env.read("s.h")
+        env.write("s", s)
+        env.execute("'s.h' @ op.zero")
+        env.execute("  ".join(words))
+        assert np.array_equal(env.read("s"), p_sep)
+        assert np.array_equal(env.read("s.h").view(np.int16), h_sep.view(np.int16))
+
+        # softmax backward straight into a 16-bit tensor
+        env.execute("%d %d %d %d 4 'cuda' 'float' op.create 'dp' !  %d %d %d %d 4 'cuda' 'float' op.create 'ds' !"
+                    % (b, h, t, t, b, h, t, t))
+        env.write("dp", rng.standard_normal((b, h, t, t)).astype(np.float32))
+        env.execute("'dp' @ 's' @ 'ds' @ op.softmax_backward  's.h' @ 'ds' @ op.copy")
+        want = env.read("s.h")
+        env.execute("'s.h' @ op.zero  'dp' @ 's' @ 's.h' @ op.softmax_backward")
+        assert np.array_equal(env.read("s.h").view(np.int16), want.view(np.int16))
     finally:
         env.close()

@@ -190,3 +190,19 @@ def test_fusion_pass_rewrites_only_push_separated_sequences(env):
     # a lone add followed by softmax is not a match
     short = "'s' @ 'm' @ 's' @ op.add  's' @ 'p' @ op.softmax"
     assert env.disassemble(short, fused=True) == env.disassemble(short)
+
+
+def test_fusion_pass_folds_a_trailing_copy_into_the_producer(env):
+    """`op.layernorm op.copy` and the score softmax followed by `op.copy`
+    become one word each; the four-word pattern wins over the three-word one,
+    which still applies when no copy follows."""
+    ln = "'x' @ 'mean' @ 'var' @ 'g' @ 'b' @ 'y' @ 1e-5 op.layernorm  'y.h' @ 'y' @ op.copy"
+    fused = env.disassemble(ln, fused=True)
+    assert [x for x in fused if x[0] in "W-"] == ["-:op.layernorm", "W:op.layernorm_copy"]
+    sm = "'s' @ 'a' @ 's' @ op.add  's' @ 'm' @ 's' @ op.add  's' @ 's' @ op.softmax"
+    with_copy = env.disassemble(sm + "  's.h' @ 's' @ op.copy", fused=True)
+    assert [x for x in with_copy if x[0] in "W-"] == ["-:op.add", "-:op.add", "-:op.softmax",
+                                                      "W:op.add_add_softmax_copy"]
+    both = env.disassemble(sm + "  's.h' @ 's' @ op.copy  " + sm + " op.sync 's.h' @ 's' @ op.copy", fused=True)
+    assert [x for x in both if x.startswith("W:")] == ["W:op.add_add_softmax_copy", "W:op.add_add_softmax",
+                                                       "W:op.sync", "W:op.copy"]
