@@ -61,6 +61,30 @@ struct Embed : public NativeWord {
     NWORD_CREATOR_DEFINE_LR(Embed)
 };
 
+// ( ids dx grad -- )  grad[ids[i], :] += dx[i, :]: the gather's backward
+struct EmbedBackward : public NativeWord {
+    void run(Stack& stack) override {
+        tensor_t grad = stack.pop_tensor();
+        tensor_t dx = stack.pop_tensor();
+        tensor_t ids = stack.pop_tensor();
+        br_assert(ids->is_cpu() && ids->dtype() == DataType::Int, "bloom.embed_backward: ids must be a cpu int tensor");
+        br_assert(grad->is_cuda() && dx->is_cuda() && grad->dtype() == DataType::Float &&
+                      dx->dtype() == DataType::Float,
+                  "bloom.embed_backward: dx and grad must be device fp32 tensors");
+        const int64_t hidden = (int64_t)grad->shape().vec().back();
+        const int64_t vocab = (int64_t)grad->items() / hidden;
+        br_assert((int64_t)dx->shape().vec().back() == hidden, "bloom.embed_backward: row lengths differ");
+        const int64_t n = (int64_t)dx->items() / hidden;
+        br_assert((int64_t)ids->items() >= n, "bloom.embed_backward: not enough ids");
+        int32_t* d_ids = static_cast<int32_t*>(ComputingContext::scratch((size_t)n * sizeof(int32_t)));
+        BR_HIP_CHECK(br_hip_memcpy_h2d(d_ids, ids->data(), (size_t)n * sizeof(int32_t), ComputingContext::stream));
+        BR_HIP_CHECK(br_hip_embedding_scatter_add(static_cast<const float*>(dx->data()), d_ids,
+                                                  static_cast<float*>(grad->data()), n, hidden, vocab,
+                                                  ComputingContext::stream));
+    }
+    NWORD_CREATOR_DEFINE_LR(EmbedBackward)
+};
+
 struct Alibi : public NativeWord {
     void run(Stack& stack) override {
         tensor_t alibi = stack.pop_tensor();
@@ -116,6 +140,7 @@ void load_bloom_words(Enviroment& env) {
     env.insert_native_word("bloom.normal", Normal::creator);
     env.insert_native_word("bloom.last_loss", LastLoss::creator);
     env.insert_native_word("bloom.embed", Embed::creator);
+    env.insert_native_word("bloom.embed_backward", EmbedBackward::creator);
     env.insert_native_word("bloom.alibi", Alibi::creator);
     env.insert_native_word("bloom.xmask", XMask::creator);
 }

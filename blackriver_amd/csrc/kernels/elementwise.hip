@@ -700,6 +700,42 @@ __global__ __launch_bounds__(kBlock) void normal_kernel(T* dst, float mean, floa
     }
 }
 
+// Backward of the row gather: grad[ids[i], :] += dx[i, :] for i = 0 .. n-1, in
+// that order, so that the result does not depend on scheduling when an id
+// occurs several times.  Workgroup i owns id = ids[i] only if i is that id's
+// first position; it then folds every later position with the same id into the
+// row, in ascending position order, starting from the row's current value.
+__global__ __launch_bounds__(kBlock) void scatter_add_rows(const float* __restrict__ dx,
+                                                            const int32_t* __restrict__ ids, float* grad, int n,
+                                                            int64_t hidden, int64_t vocab, bool vec) {
+    const int i = blockIdx.x;
+    const int32_t id = ids[i];
+    if (id < 0 || (int64_t)id >= vocab) return;
+    int seen = 0;
+    for (int j = threadIdx.x; j < i; j += kBlock) seen |= ids[j] == id;
+    if (__syncthreads_or(seen)) return;
+    float* row = grad + (int64_t)id * hidden;
+    if (vec) {
+        const int64_t h4 = hidden / 4;
+        for (int64_t c = threadIdx.x; c < h4; c += kBlock) {
+            float4 acc = reinterpret_cast<float4*>(row)[c];
+            for (int j = i; j < n; j++) {
+                if (ids[j] != id) continue;
+                const float4 d = reinterpret_cast<const float4*>(dx + (int64_t)j * hidden)[c];
+                acc.x += d.x; acc.y += d.y; acc.z += d.z; acc.w += d.w;
+            }
+            reinterpret_cast<float4*>(row)[c] = acc;
+        }
+    } else {
+        for (int64_t c = threadIdx.x; c < hidden; c += kBlock) {
+            float acc = row[c];
+            for (int j = i; j < n; j++)
+                if (ids[j] == id) acc += dx[(int64_t)j * hidden + c];
+            row[c] = acc;
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -1064,6 +1100,18 @@ int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, in
     else
         gather_rows_bytes<<<(unsigned)n, kBlock, 0, st>>>((const unsigned char*)table, ids, (unsigned char*)out,
                                                           row_bytes, vocab);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_embedding_scatter_add(const float* dx, const int32_t* ids, float* grad, int64_t n, int64_t hidden,
+                                 int64_t vocab, br_stream_t stream) {
+    if (n < 0 || hidden <= 0 || vocab <= 0 || n > 0x7fffffff) return BR_ERR_ATTR;
+    if (n == 0) return BR_OK;
+    if (!dx || !ids) return BR_ERR_INPUT;
+    if (!grad || (const float*)grad == dx) return BR_ERR_OUTPUT;
+    const bool vec = hidden % 4 == 0 && aligned16(dx) && aligned16(grad);
+    scatter_add_rows<<<(unsigned)n, kBlock, 0, as_stream(stream)>>>(dx, ids, grad, (int)n, hidden, vocab, vec);
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }

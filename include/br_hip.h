@@ -291,6 +291,13 @@ int br_hip_probe_mfma_f16(int random_operands, int passes, float* scratch, int64
 /* The embedding row gather of blackriver/train_bloom.cpp:50-56. */
 int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, int elem_bytes,
                             int64_t n, int64_t hidden, int64_t vocab, br_stream_t stream);
+/* Backward of that gather: grad[ids[i], :] += dx[i, :] for i = 0 .. n-1 in
+ * ascending i (fp32; repeated ids are summed in position order, so the result
+ * is deterministic); ids outside [0, vocab) are skipped.  The reference has no
+ * embedding gradient (its table is frozen, train.words:264-268 only gathers);
+ * with the LM head tied to the table this completes the table's gradient. */
+int br_hip_embedding_scatter_add(const float* dx, const int32_t* ids, float* grad, int64_t n,
+                                 int64_t hidden, int64_t vocab, br_stream_t stream);
 /* The ALiBi table of train_bloom.cpp:58-71: alibi[h,k] = (float)(k*slope_h),
  * slope_h = (2^(-2^(3-log2 heads)))^(h+1) evaluated in fp64 on the host. */
 int br_hip_alibi_table(float* alibi, int64_t heads, int64_t tokens, br_stream_t stream);

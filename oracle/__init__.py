@@ -314,6 +314,15 @@ def embedding_gather(vocab, ids):
     return out
 
 
+def embedding_scatter_add(grad, dx, ids):
+    """grad[ids[i]] += dx[i] in ascending i, in place on a copy; returns it."""
+    grad = np.array(_f(grad), copy=True)
+    dx, ids = _f(dx), _i(ids)
+    lib().orc_embedding_scatter_add(_p(grad), _p(dx), _p(ids), _i64(ids.size), _i64(grad.shape[1]),
+                                    _i64(grad.shape[0]))
+    return grad
+
+
 def alibi(heads, tokens):
     out = np.empty((heads, tokens), np.float32)
     lib().orc_alibi(_p(out), _i64(heads), _i64(tokens))

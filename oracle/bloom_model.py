@@ -2,7 +2,8 @@
 everything under oracle/): embedding gather + embedding LayerNorm, N decoder
 blocks, final LayerNorm, LM-head loss, and the backward chain, composed from
 the operator restatements exactly as BlackRiver's model script composes them
-(bloomz-7b/train.words:250-318 for rank 0's head and tail, :137-248 per block).
+(bloomz-7b/train.words:250-318 for rank 0's head and tail, :137-248 per block),
+plus the gradient of the embedding table, which the reference keeps frozen.
 
 Pinned by: the per-operator checks of the functions it calls, and a central
 finite difference of the whole loss with respect to a few weights
@@ -47,5 +48,7 @@ def model_step(model_w, layer_ws, ids, mask, heads, eps=1e-5):
     dx, g0["word_embeddings_layernorm.weight_g"], g0["word_embeddings_layernorm.bias_g"] = orc.layernorm_bwd(
         dx, emb_y, model_w["word_embeddings_layernorm.weight"], model_w["word_embeddings_layernorm.bias"], emb_var, eps)
     g0["embedding_rows_g"] = dx
+    # the table is tied: its gradient is the head's plus the scatter of the row gradients
+    g0["word_embeddings.weight_g"] = orc.embedding_scatter_add(head_g, dx.reshape(-1, h), ids.reshape(-1))
     grads[0] = g0
     return loss, grads

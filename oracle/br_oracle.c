@@ -518,6 +518,18 @@ void orc_embedding_gather(const float* vocab, const int32_t* ids, float* out,
                sizeof(float) * (size_t)hidden);
 }
 
+/* Backward of the gather (no counterpart in the reference, whose embedding
+ * table is frozen): the plain sequential scatter, which fixes the summation
+ * order for repeated ids. */
+void orc_embedding_scatter_add(float* grad, const float* dx, const int32_t* ids,
+                               int64_t n, int64_t hidden, int64_t vocab) {
+    for (int64_t i = 0; i < n; i++) {
+        if (ids[i] < 0 || ids[i] >= vocab) continue;
+        float* row = grad + (int64_t)ids[i] * hidden;
+        for (int64_t c = 0; c < hidden; c++) row[c] += dx[i * hidden + c];
+    }
+}
+
 void orc_alibi(float* alibi, int64_t heads, int64_t tokens) {
     double base = 3 - log2((double)heads * 1.0);
     base = -1 * pow(2.0, base);

@@ -133,6 +133,11 @@ float orc_logsoftmax_nll(const float* logits, const int32_t* target,
 /* blackriver/train_bloom.cpp:50-56 */
 void orc_embedding_gather(const float* vocab, const int32_t* ids, float* out,
                           int64_t n, int64_t hidden);
+/* Backward of the gather: grad[ids[i],:] += dx[i,:], i ascending.  Not in the
+ * reference (frozen table); pinned by autograd of the tied table in
+ * tests/test_oracle_model.py and by brute force in tests/test_oracle_ops.py. */
+void orc_embedding_scatter_add(float* grad, const float* dx, const int32_t* ids,
+                               int64_t n, int64_t hidden, int64_t vocab);
 /* train_bloom.cpp:58-71 */
 void orc_alibi(float* alibi, int64_t heads, int64_t tokens);
 /* train_bloom.cpp:73-90 */

@@ -249,3 +249,22 @@ def test_xmask_table_bit_exact(fixture_ids_mask):
     out2 = empty((3, 5, 5))
     call("br_hip_xmask_table", ptr(dev(holes)), ptr(out2), 3, 5, stream())
     assert np.array_equal(host(out2), orc.xmask(holes))
+
+
+@pytest.mark.parametrize("n,hidden,vocab", [(2048, 4096, 512), (37, 100, 11), (64, 256, 1), (5, 8, 1000)])
+def test_embedding_scatter_add_is_the_sequential_scatter(n, hidden, vocab):
+    """Backward of the embedding gather: bit-exact against the oracle's
+    sequential loop (repeated ids are summed in position order), with many
+    repeats (vocab < n), a single row taking everything (vocab 1), ids outside
+    the table skipped, and a non-zero starting gradient."""
+    print("case n=%d hidden=%d vocab=%d" % (n, hidden, vocab), flush=True)
+    rng = np.random.default_rng(31)
+    ids = rng.integers(0, vocab, n).astype(np.int32)
+    if n > 4:
+        ids[1], ids[3] = -1, vocab       # outside the table
+    dx = rng.standard_normal((n, hidden)).astype(np.float32)
+    grad = rng.standard_normal((vocab, hidden)).astype(np.float32)
+    want = orc.embedding_scatter_add(grad, dx, ids)
+    d_grad = dev(grad)
+    call("br_hip_embedding_scatter_add", ptr(dev(dx)), ptr(dev(ids)), ptr(d_grad), n, hidden, vocab, stream())
+    assert np.array_equal(host(d_grad), want)

@@ -66,9 +66,11 @@ def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden,
                     continue
                 assert_close(model.read(i, name + "_g"), ref[i][name + "_g"], tol, "block %d %s_g" % (i, name))
         for name in ("ln_f.weight", "ln_f.bias", "word_embeddings_layernorm.weight",
-                     "word_embeddings_layernorm.bias", "lm_head.weight"):
+                     "word_embeddings_layernorm.bias", "word_embeddings.weight"):
             assert_close(model.read(0, name + "_g"), ref[0][name + "_g"], tol, name + "_g")
         assert_close(model.read(0, "xc"), ref[0]["embedding_rows_g"], tol, "gradient of the embedding rows")
+        # the head is tied to the table: one gradient tensor under both names
+        assert np.array_equal(model.read(0, "lm_head.weight_g"), model.read(0, "word_embeddings.weight_g"))
         # a second step on the same batch: gradients are overwritten, the head's
         # accumulator is cleared, so everything repeats exactly
         g1 = model.read(0, "lm_head.weight_g")

@@ -65,3 +65,5 @@ def test_model_step_against_textbook_autograd():
     head = mt["word_embeddings.weight"].grad.numpy().copy()
     np.subtract.at(head, ids.reshape(-1), rows.grad.numpy().reshape(-1, h))
     assert_close(grads[0]["lm_head.weight_g"], head, 2e-4, "lm_head gradient")
+    assert_close(grads[0]["word_embeddings.weight_g"], mt["word_embeddings.weight"].grad.numpy(), 2e-4,
+                 "tied table gradient")

@@ -299,3 +299,27 @@ def test_f16_converters_match_numpy_bit_for_bit():
     with np.errstate(over="ignore"):
         want = x.astype(np.float16).view(np.uint16)
     assert np.array_equal(orc.f32_to_f16_bits(x), want)
+
+
+def test_embedding_scatter_add_against_brute_force_and_numpy():
+    """grad[ids[i]] += dx[i] in ascending i: the same as numpy's unbuffered
+    np.add.at (also sequential, hence bit-exact) and, within rounding, as the
+    one-hot matrix product onehot(ids)^T . dx; ids outside the table are skipped."""
+    rng = np.random.default_rng(9)
+    n, hidden, vocab = 50, 12, 7
+    ids = rng.integers(0, vocab, n).astype(np.int32)
+    dx = rng.standard_normal((n, hidden)).astype(np.float32)
+    grad = rng.standard_normal((vocab, hidden)).astype(np.float32)
+    got = orc.embedding_scatter_add(grad, dx, ids)
+    want = grad.copy()
+    np.add.at(want, ids, dx)
+    assert np.array_equal(got, want)
+    onehot = np.zeros((n, vocab))
+    onehot[np.arange(n), ids] = 1
+    assert_close(got, grad + onehot.T @ dx.astype(np.float64), 1e-5, "one-hot product")
+    bad = ids.copy()
+    bad[0], bad[1] = -3, vocab
+    got = orc.embedding_scatter_add(grad, dx, bad)
+    want = grad.copy()
+    np.add.at(want, bad[2:], dx[2:])
+    assert np.array_equal(got, want)
