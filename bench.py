@@ -280,6 +280,20 @@ def elementwise_leg(hip, timer, torch):
     sec = timer.run(lambda i: hip.call("br_hip_logsoftmax_nll_bwd", vp(logits), vp(target), vp(keep), vp(lse), vp(dl),
                                        hip.F32, 1.0 / rows, rows, vocab, st), 20, 3)
     rec("logsoftmax_nll_bwd [2048,250880] f32", sec, 2 * rows * vocab * 4)
+    del logits, dl
+
+    # AdamW over one h -> 4h matrix (fp16 parameter with fp32 master copy):
+    # reads grad, m, v, master (16 B), writes m, v, master (12 B) and the fp16 parameter (2 B)
+    n = 4 * 4096 * 4096
+    ps = [torch.zeros(n, device="cuda", dtype=torch.float16) for _ in range(2)]
+    ms = [torch.randn(n, device="cuda") * 0.02 for _ in range(2)]
+    gs = [torch.randn(n, device="cuda") for _ in range(2)]
+    m1 = [torch.zeros(n, device="cuda") for _ in range(2)]
+    m2 = [torch.zeros(n, device="cuda") for _ in range(2)]
+    sec = timer.run(lambda i: hip.call("br_hip_adamw", vp(ps[i % 2]), hip.F16, vp(ms[i % 2]), vp(gs[i % 2]),
+                                       vp(m1[i % 2]), vp(m2[i % 2]), n, 1e-4, 0.9, 0.95, 1e-8, 0.01, 1 + i // 2, st),
+                    40, 4)
+    rec("adamw [16384,4096] f16 + f32 master", sec, 30 * n)
     return out
 
 

@@ -111,6 +111,36 @@ void BloomTrainer::init_synthetic(uint64_t seed, float std) {
     env_.execute(s.str());
 }
 
+void BloomTrainer::create_optimizer(float lr, float beta1, float beta2, float eps, float weight_decay) {
+    br_assert(step_ != nullptr, "BloomTrainer::create has not run");
+    br_assert(!has_optimizer_, "the optimizer state exists already");
+    std::ostringstream s;
+    s.precision(9);
+    for (int i = 0; i <= cfg_.layers; i++) {
+        s << i << " #  " << lr << " " << beta1 << " " << beta2 << " " << eps << " " << weight_decay << " adamw_hyper\n";
+        s << (i == 0 ? "create_model_adamw" : "create_layer_adamw");
+        if (masters()) s << (i == 0 ? " create_model_masters" : " create_layer_masters");
+        s << "\n";
+    }
+    s << "0 # op.sync\n";
+    env_.execute(s.str());
+    has_optimizer_ = true;
+    adam_step_ = 0;
+}
+
+void BloomTrainer::optimizer_step() {
+    br_assert(has_optimizer_, "BloomTrainer::create_optimizer has not run");
+    adam_step_++;
+    // the step count changes every call, so the (short) program is compiled per call
+    std::ostringstream s;
+    const char* sfx = masters() ? "16" : "";
+    s << "0 #  " << adam_step_ << " $adam_step !  model_adamw" << sfx << "\n";
+    for (int i = 1; i <= cfg_.layers; i++)
+        s << i << " #  " << adam_step_ << " $adam_step !  layer_adamw" << sfx << "\n";
+    s << "0 # op.sync\n";
+    env_.execute(s.str());
+}
+
 float BloomTrainer::step(const int32_t* ids, const int32_t* mask) {
     br_assert(step_ != nullptr, "BloomTrainer::create has not run");
     env_.change(0);

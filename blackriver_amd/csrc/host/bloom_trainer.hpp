@@ -39,6 +39,14 @@ public:
     // mean log-probability of the labels (the sign convention of op.loss_backward).
     float step(const int32_t* ids, const int32_t* mask);
 
+    // AdamW state for every parameter (moments; fp32 master copies of 16-bit
+    // matrices, initialised from the matrices as they are now: call after the
+    // weights have their starting values).
+    void create_optimizer(float lr, float beta1, float beta2, float eps, float weight_decay);
+    // One AdamW step over every parameter from the gradients of the last step().
+    void optimizer_step();
+    int64_t optimizer_steps() const { return adam_step_; }
+
     const BloomModelConfig& config() const { return cfg_; }
     // floats of a block's arena / of hash 0's arena (which ends in the logits rows)
     int64_t block_arena_floats() const;
@@ -51,6 +59,9 @@ private:
     Enviroment& env_;
     BloomModelConfig cfg_;
     std::unique_ptr<DaG> step_;
+    bool masters() const { return cfg_.weight_dtype != "float"; }
+    bool has_optimizer_ = false;
+    int64_t adam_step_ = 0;
 };
 
 }  // namespace br

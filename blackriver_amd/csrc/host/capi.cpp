@@ -299,6 +299,20 @@ int br_bloom_model_step(br_env_t* e, const int32_t* ids, const int32_t* mask, fl
     });
 }
 
+int br_bloom_model_optimizer_create(br_env_t* e, float lr, float beta1, float beta2, float eps, float weight_decay) {
+    return guarded([&]() {
+        br_assert(e->trainer != nullptr, "br_bloom_model_create has not run");
+        e->trainer->create_optimizer(lr, beta1, beta2, eps, weight_decay);
+    });
+}
+
+int br_bloom_model_optimizer_step(br_env_t* e) {
+    return guarded([&]() {
+        br_assert(e->trainer != nullptr, "br_bloom_model_create has not run");
+        e->trainer->optimizer_step();
+    });
+}
+
 int br_bloom_fetch_data(const int32_t* ids, const int32_t* mask, int64_t batch, int64_t tokens, const float* vocab,
                         int64_t hidden, int64_t heads, float* xinput, float* alibi, float* xmask) {
     return guarded([&]() {

@@ -215,6 +215,39 @@ BR_WORD(SoftmaxAttnBackward, Tensors<5> a(stack); a[0]->op_softmax_attn_backward
 // ( dS q k q_g k_g -- )
 BR_WORD(QueryKeyBackward, Tensors<5> a(stack); a[0]->op_qk_backward(a[0], a[1], a[2], a[3], a[4]);)
 
+// AdamW on one parameter tensor.  The reference stops at the gradients; these
+// two words are what a training loop runs after them.
+// ( param [master] grad m v lr beta1 beta2 eps weight_decay step -- )
+void adamw(Stack& stack, bool with_master) {
+    const double step = stack.pop_number();
+    const float wd = (float)stack.pop_number();
+    const float eps = (float)stack.pop_number();
+    const float beta2 = (float)stack.pop_number();
+    const float beta1 = (float)stack.pop_number();
+    const float lr = (float)stack.pop_number();
+    tensor_t v = stack.pop_tensor();
+    tensor_t m = stack.pop_tensor();
+    tensor_t grad = stack.pop_tensor();
+    tensor_t master = with_master ? stack.pop_tensor() : nullptr;
+    tensor_t param = stack.pop_tensor();
+    auto f32dev = [](const tensor_t& x) { return x->is_cuda() && x->dtype() == DataType::Float; };
+    br_assert(param->is_cuda() && f32dev(grad) && f32dev(m) && f32dev(v), "op.adamw: device tensors, fp32 state");
+    br_assert(grad->items() == param->items() && m->items() == param->items() && v->items() == param->items(),
+              "op.adamw: parameter, gradient and moments differ in size");
+    br_assert(step >= 1, "op.adamw: steps count from 1");
+    float* master_ptr = nullptr;
+    if (with_master) {
+        br_assert(f32dev(master) && master->items() == param->items() && param->dtype() != DataType::Float,
+                  "op.adamw_master: an fp32 master copy of a 16-bit parameter");
+        master_ptr = static_cast<float*>(master->data());
+    }
+    BR_HIP_CHECK(br_hip_adamw(param->data(), (int)param->dtype(), master_ptr, static_cast<const float*>(grad->data()),
+                              static_cast<float*>(m->data()), static_cast<float*>(v->data()), (int64_t)param->items(),
+                              lr, beta1, beta2, eps, wd, (int64_t)step, ComputingContext::stream));
+}
+BR_WORD(AdamW, adamw(stack, false);)
+BR_WORD(AdamWMaster, adamw(stack, true);)
+
 BR_WORD(Dump, tensor_t t = stack.pop_tensor(); t->io_dump(t);)
 // ( tensor filename -- )
 BR_WORD(Load, const std::string f = stack.pop_string(); tensor_t t = stack.pop_tensor(); t->io_load(t, f.c_str());)
@@ -266,6 +299,8 @@ void load_nn_words(Enviroment& env) {
         {"op.softmax_backward", SoftmaxBackward::creator},
         {"op.softmax_attn_backward", SoftmaxAttnBackward::creator},
         {"op.qk_backward", QueryKeyBackward::creator},
+        {"op.adamw", AdamW::creator},
+        {"op.adamw_master", AdamWMaster::creator},
     };
     for (const auto& e : table) env.insert_native_word(e.name, e.creator);
     // longer patterns first: a pass only sees what earlier passes left unfused

@@ -55,6 +55,8 @@ SIGNATURES = {
     "br_bloom_model_create": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _i64, ctypes.c_float, _cp, _cp]),
     "br_bloom_model_init": (_int, [_vp, ctypes.c_uint64, ctypes.c_float]),
     "br_bloom_model_step": (_int, [_vp, _i32p, _i32p, ctypes.POINTER(ctypes.c_float)]),
+    "br_bloom_model_optimizer_create": (_int, [_vp] + [ctypes.c_float] * 5),
+    "br_bloom_model_optimizer_step": (_int, [_vp]),
     "br_bloom_fetch_data": (_int, [_i32p, _i32p, _i64, _i64, _f32p, _i64, _i64, _f32p, _f32p, _f32p]),
 }
 
@@ -264,6 +266,15 @@ class BloomModel:
         _check(load().br_bloom_model_step(self.env._h, ids.ctypes.data_as(_i32p), mask.ctypes.data_as(_i32p),
                                           ctypes.byref(loss)), "model_step")
         return loss.value
+
+    def create_optimizer(self, lr=1e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.0):
+        """AdamW state (moments, fp32 masters of 16-bit matrices).  Call after
+        the weights have their starting values."""
+        _check(load().br_bloom_model_optimizer_create(self.env._h, lr, beta1, beta2, eps, weight_decay),
+               "optimizer_create")
+
+    def optimizer_step(self):
+        _check(load().br_bloom_model_optimizer_step(self.env._h), "optimizer_step")
 
     def read(self, layer, name):
         self.env.change_hash(layer)

@@ -277,6 +277,20 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
                        const float* bias, int64_t batch, int compute,
                        void* workspace, size_t workspace_bytes, br_stream_t stream);
 
+/* ---- optimizer ---------------------------------------------------------- */
+/* One AdamW step (decoupled weight decay) over n parameters, all arithmetic in
+ * fp32:  p *= 1 - lr*wd;  m += (g - m)(1 - beta1);  v = beta2 v + (1 - beta2) g^2;
+ * p -= lr / (1 - beta1^step) * m / (sqrt(v) / sqrt(1 - beta2^step) + eps).
+ * param_dtype BR_F32: master must be NULL, the parameter is updated in place.
+ * BR_F16 / BR_BF16: with an fp32 `master` copy the master is updated and param
+ * receives its rounding; without one the 16-bit value itself is the state.
+ * step counts from 1.  The reference has no optimizer (its training loop stops
+ * at the gradients, bloomz-7b/train.words:320-366); this is what a training
+ * run needs after them. */
+int br_hip_adamw(void* param, int param_dtype, float* master, const float* grad, float* m, float* v,
+                 int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
+                 int64_t step, br_stream_t stream);
+
 /* ---- calibration ------------------------------------------------------- */
 /* Rate of a bare v_mfma_f32_32x32x16_f16 loop without any memory traffic, with
  * operands of zeros (random_operands == 0) or of random values: on MI355X the

@@ -101,6 +101,14 @@ int br_bloom_model_create(br_env_t* env, int layers, int64_t batch, int64_t toke
                           const char* gemm_precision);
 int br_bloom_model_init(br_env_t* env, uint64_t seed, float std);
 int br_bloom_model_step(br_env_t* env, const int32_t* ids, const int32_t* mask, float* loss);
+/* AdamW over every parameter of the model (the reference's loop ends at the
+ * gradients, bloomz-7b/train.words:320-366).  optimizer_create allocates the
+ * moments and, for 16-bit matrices, fp32 master copies initialised from the
+ * matrices as they are at that moment; optimizer_step applies one update from
+ * the gradients the last br_bloom_model_step left. */
+int br_bloom_model_optimizer_create(br_env_t* env, float lr, float beta1, float beta2, float eps,
+                                    float weight_decay);
+int br_bloom_model_optimizer_step(br_env_t* env);
 
 /* The host-side batch preparation of BloomInput::fetch_data
  * (train_bloom.cpp:41-93) on caller-provided host buffers:

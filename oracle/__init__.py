@@ -350,3 +350,21 @@ def f16_bits_to_f32(x):
     y = np.empty(x.shape, np.float32)
     lib().orc_f16_to_f32(_p(x), _p(y), _i64(x.size))
     return y
+
+
+def adamw_step(param, grad, m, v, lr, beta1, beta2, eps, weight_decay, step):
+    """One AdamW step in fp32, operation for operation the single-tensor update
+    of torch.optim.AdamW (decoupled decay, lerp for the first moment, bias
+    corrections from python floats).  The reference has no optimizer; pinned
+    against torch.optim.AdamW itself in tests/test_oracle_ops.py.
+    Returns (param, m, v) as new fp32 arrays."""
+    f = np.float32
+    p = _f(param) * f(1.0 - lr * weight_decay)
+    g = _f(grad)
+    m = _f(m) + (g - _f(m)) * f(1.0 - beta1)
+    v = _f(v) * f(beta2) + (f(1.0 - beta2) * g) * g
+    bc1 = 1.0 - beta1 ** step
+    bc2 = 1.0 - beta2 ** step
+    denom = np.sqrt(v) / f(bc2 ** 0.5) + f(eps)
+    p = p - f(lr / bc1) * (m / denom)
+    return p.astype(np.float32), m.astype(np.float32), v.astype(np.float32)

@@ -248,3 +248,36 @@ def test_device_tensor_plumbing(runtime, tmp_path, capfd):
     with pytest.raises(host.HostError, match="same size"):
         env.execute("1024 1 'cuda' 'float' op.create '%s' io.load" % f)
     env.close()
+
+
+@pytest.mark.parametrize("dtype", ["float", "f16"])
+def test_qkv_relayout_words_match_the_offline_converter(runtime, dtype):
+    """qkv_*_from_hf reorder the rows of a Hugging Face fused query_key_value
+    tensor, [head, q|k|v, d], into BlackRiver's [q|k|v, head, d]: the view /
+    transpose / reshape of bloomz-7b/dump_weights.py:23-44, restated here with
+    numpy.  qkv_*_to_hf is the inverse.  Pure data movement: exact."""
+    hidden, heads = 256, 4
+    hd = hidden // heads
+    rng = np.random.default_rng(2)
+    env = host.Env(1)
+    try:
+        env.execute(host.words_text("bloom.words"))
+        env.execute("%d %d 1024 1e-05 model_dims" % (hidden, heads))
+        for name, shape in (("w", "%d %d 2" % (3 * hidden, hidden)), ("b", "%d 1" % (3 * hidden))):
+            for sfx in (".hf", "", ".back"):
+                env.execute("%s 'cuda' '%s' op.create '%s%s' !" % (shape, dtype, name, sfx))
+        w = rng.standard_normal((3 * hidden, hidden)).astype(np.float16).astype(np.float32)
+        b = rng.standard_normal(3 * hidden).astype(np.float16).astype(np.float32)
+        env.write("w.hf", w)
+        env.write("b.hf", b)
+        env.execute("'w.hf' @ 'w' @ qkv_weight_from_hf   'b.hf' @ 'b' @ qkv_bias_from_hf")
+        want_w = w.reshape(heads, 3, hd, hidden).transpose(1, 0, 2, 3).reshape(3 * hidden, hidden)
+        want_b = b.reshape(heads, 3, hd).transpose(1, 0, 2).reshape(3 * hidden)
+        assert np.array_equal(env.read("w"), want_w)
+        assert np.array_equal(env.read("b"), want_b)
+        # the first third is the query projection of every head, heads in order
+        assert np.array_equal(env.read("w")[:hd], w[:hd]) and np.array_equal(env.read("w")[hd:2 * hd], w[3 * hd:4 * hd])
+        env.execute("'w' @ 'w.back' @ qkv_weight_to_hf   'b' @ 'b.back' @ qkv_bias_to_hf")
+        assert np.array_equal(env.read("w.back"), w) and np.array_equal(env.read("b.back"), b)
+    finally:
+        env.close()

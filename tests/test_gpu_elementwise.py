@@ -9,7 +9,7 @@ import torch
 
 import oracle as orc
 from conftest import assert_close
-from gpu_util import (F16, F32, I32, assert_close_f16, call, dev, empty, host, ptr, stream, workspace)
+from gpu_util import (BF16, F16, F32, I32, assert_close_f16, call, dev, empty, host, ptr, stream, workspace)
 from blackriver_amd import hip
 
 pytestmark = pytest.mark.gpu
@@ -268,3 +268,51 @@ def test_embedding_scatter_add_is_the_sequential_scatter(n, hidden, vocab):
     d_grad = dev(grad)
     call("br_hip_embedding_scatter_add", ptr(dev(dx)), ptr(dev(ids)), ptr(d_grad), n, hidden, vocab, stream())
     assert np.array_equal(host(d_grad), want)
+
+
+@pytest.mark.parametrize("dtype,master", [(F32, False), (F16, True), (F16, False), (BF16, True)])
+@pytest.mark.parametrize("n", [4096 * 1024, 1001])
+def test_adamw_against_oracle(n, dtype, master):
+    """Three AdamW steps against the oracle's fp32 restatement (itself pinned to
+    torch.optim.AdamW): parameter / master and both moments within 1e-5; a
+    16-bit parameter is exactly the rounding of its master copy."""
+    print("case n=%d dtype=%d master=%s" % (n, dtype, master), flush=True)
+    rng = np.random.default_rng(17)
+    tdt = {F32: torch.float32, F16: torch.float16, BF16: torch.bfloat16}[dtype]
+    p0 = torch.from_numpy(rng.standard_normal(n).astype(np.float32)).to(tdt)
+    d_p = p0.cuda()
+    d_master = p0.float().cuda() if master else None
+    d_m, d_v = torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    p, m, v = p0.float().numpy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    lr, b1, b2, eps, wd = 1e-2, 0.9, 0.95, 1e-8, 0.1
+    for step in range(1, 4):
+        g = rng.standard_normal(n).astype(np.float32)
+        call("br_hip_adamw", ptr(d_p), dtype, ptr(d_master), ptr(dev(g)), ptr(d_m), ptr(d_v), n, lr, b1, b2, eps, wd,
+             step, stream())
+        p, m, v = orc.adamw_step(p, g, m, v, lr, b1, b2, eps, wd, step)
+        assert_close(host(d_m), m, 1e-5, "first moment, step %d" % step)
+        assert_close(host(d_v), v, 1e-5, "second moment, step %d" % step)
+        if dtype == F32:
+            assert_close(host(d_p), p, 1e-5, "parameter, step %d" % step)
+        elif master:
+            assert_close(host(d_master), p, 1e-5, "master copy, step %d" % step)
+            assert torch.equal(d_p, d_master.to(tdt))
+        else:
+            # the 16-bit value is the only state: the oracle follows the same rounding
+            p = torch.from_numpy(p).to(tdt).float().numpy()
+            got = host(d_p.float())
+            ulp = np.abs(p) * (2.0 ** -10 if dtype == F16 else 2.0 ** -7)
+            assert np.all(np.abs(got - p) <= ulp + 1e-6)
+            p = got
+
+
+def test_adamw_rejects_bad_arguments():
+    lib = hip.load()
+    t = empty(16)
+    args = (16, 1e-3, 0.9, 0.95, 1e-8, 0.0)
+    assert lib.br_hip_adamw(ptr(t), F32, ptr(t), ptr(t), ptr(t), ptr(t), *args, 1, stream()) == -4   # fp32 + master
+    assert lib.br_hip_adamw(ptr(t), F32, None, ptr(t), ptr(t), ptr(t), *args, 0, stream()) == -4      # step from 1
+    assert lib.br_hip_adamw(ptr(t), F32, None, None, ptr(t), ptr(t), *args, 1, stream()) == -2
+    assert lib.br_hip_adamw(None, F32, None, ptr(t), ptr(t), ptr(t), *args, 1, stream()) == -3
+    assert lib.br_hip_adamw(ptr(t), I32, None, ptr(t), ptr(t), ptr(t), *args, 1, stream()) == -1
+    torch.cuda.synchronize()

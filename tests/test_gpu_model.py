@@ -10,6 +10,7 @@ the GPU by the C++ driver, compared with the CPU oracle's composition
 import numpy as np
 import pytest
 
+import oracle as orc
 from oracle import bloom_block as blk
 from oracle import bloom_model as mdl
 from conftest import assert_close
@@ -79,5 +80,47 @@ def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden,
         assert loss2 == loss
         assert np.array_equal(model.read(0, "lm_head.weight_g"), g1)
         assert np.array_equal(model.read(1, "dense.weight_g"), d1)
+    finally:
+        model.close()
+
+
+@pytest.mark.parametrize("mode", ["fp32", "f16"])
+def test_adamw_updates_every_parameter_and_training_raises_the_log_probability(runtime, mode):
+    """After one step + optimizer step every parameter tensor equals the
+    oracle's AdamW applied to the gradients the device holds (wiring: names,
+    master copies, step count); repeating on one batch raises the mean
+    log-probability of its labels."""
+    layers, batch, tokens, hidden, heads, vocab = 2, 2, 32, 256, 4, 512
+    model, model_w, layer_ws, ids, mask = build(mode, layers, batch, tokens, hidden, heads, vocab, seed=9)
+    lr, b1, b2, eps, wd = 2e-3, 0.9, 0.95, 1e-8, 0.01
+    names0 = ["word_embeddings.weight", "word_embeddings_layernorm.weight", "word_embeddings_layernorm.bias",
+              "ln_f.weight", "ln_f.bias"]
+    names_i = ["input_layernorm.weight", "input_layernorm.bias", "post_attention_layernorm.weight",
+               "post_attention_layernorm.bias", "query_key_value.weight", "query_key_value.bias", "dense.weight",
+               "dense.bias", "dense_h_to_4h.weight", "dense_h_to_4h.bias", "dense_4h_to_h.weight", "dense_4h_to_h.bias"]
+    every = [(0, n) for n in names0] + [(i, n) for i in range(1, layers + 1) for n in names_i]
+    try:
+        model.create_optimizer(lr, b1, b2, eps, wd)
+        before = {k: model.read(*k) for k in every}
+        first = model.step(ids, mask)
+        model.optimizer_step()
+        for k in every:
+            g = model.read(k[0], k[1] + "_g")
+            want, m, v = orc.adamw_step(before[k], g, np.zeros_like(g), np.zeros_like(g), lr, b1, b2, eps, wd, 1)
+            got = model.read(*k)
+            assert not np.array_equal(got, before[k]), k
+            matrix16 = mode == "f16" and k[1].endswith(".weight") and "layernorm" not in k[1] and "ln_f" not in k[1]
+            if matrix16:
+                assert_close(model.read(k[0], k[1] + "_w32"), want, 1e-5, "%d %s master" % k)
+                assert np.array_equal(got, model.read(k[0], k[1] + "_w32").astype(np.float16).astype(np.float32))
+            else:
+                assert_close(got, want, 1e-5, "%d %s" % k)
+            assert_close(model.read(k[0], k[1] + "_m"), m, 1e-5, "%d %s first moment" % k)
+        losses = [first]
+        for _ in range(8):
+            losses.append(model.step(ids, mask))
+            model.optimizer_step()
+        assert losses[-1] > losses[0] + 0.5, losses      # log-probability rises
+        assert all(np.isfinite(losses))
     finally:
         model.close()

@@ -323,3 +323,28 @@ def test_embedding_scatter_add_against_brute_force_and_numpy():
     want = grad.copy()
     np.add.at(want, bad[2:], dx[2:])
     assert np.array_equal(got, want)
+
+
+def test_adamw_step_against_torch_optim():
+    """The oracle's AdamW restatement against torch.optim.AdamW on the CPU over
+    several steps (so the bias corrections and the moment recurrences are
+    exercised), with weight decay on and off."""
+    rng = np.random.default_rng(4)
+    for wd in (0.0, 0.1):
+        p0 = rng.standard_normal(1000).astype(np.float32)
+        tp = torch.nn.Parameter(torch.from_numpy(p0.copy()))
+        opt = torch.optim.AdamW([tp], lr=3e-3, betas=(0.9, 0.95), eps=1e-8, weight_decay=wd)
+        p, m, v = p0, np.zeros_like(p0), np.zeros_like(p0)
+        for step in range(1, 6):
+            g = (rng.standard_normal(1000) * 10.0 ** int(rng.integers(-3, 2))).astype(np.float32)
+            tp.grad = torch.from_numpy(g.copy())
+            opt.step()
+            p, m, v = orc.adamw_step(p, g, m, v, 3e-3, 0.9, 0.95, 1e-8, wd, step)
+            assert_close(p, tp.detach().numpy(), 1e-6, "parameter after step %d" % step)
+            st = opt.state[tp]
+            assert_close(m, st["exp_avg"].numpy(), 1e-6, "first moment")
+            assert_close(v, st["exp_avg_sq"].numpy(), 1e-6, "second moment")
+    # a plain descent direction: positive gradient lowers the parameter
+    p, _, _ = orc.adamw_step(np.ones(4, np.float32), np.ones(4, np.float32), np.zeros(4), np.zeros(4), 1e-2, 0.9,
+                             0.999, 1e-8, 0.0, 1)
+    assert np.all(p < 1.0) and np.allclose(p, 1.0 - 1e-2, rtol=1e-5)
