@@ -277,6 +277,28 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
                        const float* bias, int64_t batch, int compute,
                        void* workspace, size_t workspace_bytes, br_stream_t stream);
 
+/* ---- fused attention --------------------------------------------------- */
+/* The operator chain of bloomz-7b/train.words:154-166 in one kernel:
+ *   o = softmax((q . k^T) / sqrt(head_dim) + alibi[h, key] + mask) . v
+ * replacing op_qk (cuda_tensor.cpp:277-330), two op_add (:206-232), op_softmax
+ * (:332-356) and op_attn (:358-398) and the [batch, heads, tokens, tokens]
+ * tensors between them.  mask(b, query, key) = 0 where key <= query and
+ * key < valid[b], else -FLT_MAX: the table of train_bloom.cpp:73-90 for a batch
+ * whose sequences are padded on the right (valid = number of real tokens; a
+ * sequence with valid == 0 gets uniform probabilities, as the chain gives).
+ * q, k, v, o: fp16 / bf16 (dtype), element (b, t, h, d) at
+ * b * batch_stride + t * row_stride + h * head_stride + d, so both
+ * [B, T, heads, 128] (the projections' own output) and [B, heads, T, 128] work.
+ * alibi: fp32 [heads, tokens] (br_hip_alibi_table); valid: device int32 [batch].
+ * lse[batch, heads, tokens] receives log sum exp of each score row, which the
+ * backward needs.  Probabilities are rounded to `dtype` before the product
+ * with v.  BR_ERR_TODO unless head_dim == 128, tokens % 4 == 0, strides % 8 == 0
+ * and 16-byte aligned bases: callers then run the unfused chain. */
+int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype, const float* alibi,
+                          const int32_t* valid, void* o, float* lse, int64_t batch, int64_t heads,
+                          int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
+                          int64_t batch_stride, br_stream_t stream);
+
 /* ---- optimizer ---------------------------------------------------------- */
 /* One AdamW step (decoupled weight decay) over n parameters, all arithmetic in
  * fp32:  p *= 1 - lr*wd;  m += (g - m)(1 - beta1);  v = beta2 v + (1 - beta2) g^2;

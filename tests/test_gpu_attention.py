@@ -1,0 +1,90 @@
+"""Fused causal ALiBi attention against the CPU oracle's chain of the unfused
+operators (scores, ALiBi add, mask add, softmax, context; and the backward
+chain), through the C ABI.  The fused kernels use fp16 / bf16 MFMA operands
+with fp32 accumulation: bound 2e-2 relative to the largest reference entry
+(the stated tolerance for 16-bit matrix products)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from conftest import assert_close
+from gpu_util import BF16, F16, call, dev, empty, host, ptr, stream
+from blackriver_amd import hip
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-2
+HD = 128
+
+
+def to16(a, tdtype):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(tdtype)
+
+
+def reference_forward(q, k, v, valid):
+    """q, k, v: fp32 [B, T, NH, HD] holding 16-bit-representable values."""
+    b, t, nh, _ = q.shape
+    mask = (np.arange(t)[None, :] < np.asarray(valid)[:, None]).astype(np.int32)
+    zq, zk, zv = (orc.transpose_0213(x) for x in (q, k, v))
+    s = orc.qk(zq, zk)
+    s = orc.add_bcast(s, orc.alibi(nh, t).reshape(1, nh, 1, t))
+    s = orc.add_bcast(s, orc.xmask(mask).reshape(b, 1, t, t))
+    p = orc.softmax_fwd(s)
+    o = orc.transpose_0213(orc.attn(p, zv))           # back to [B, T, NH, HD]
+    return o, p, (zq, zk, zv)
+
+
+@pytest.mark.parametrize("dtype,tdtype", [(F16, torch.float16), (BF16, torch.bfloat16)])
+@pytest.mark.parametrize("b,nh,t,valid", [
+    (2, 4, 512, (512, 300)),      # the block's sequence length, one padded sequence
+    (1, 2, 64, (64,)),
+    (2, 3, 200, (200, 1)),        # tokens not a multiple of the tile sizes; a one-token sequence
+    (2, 2, 132, (0, 77)),         # an empty sequence: uniform probabilities, as the unfused chain gives
+    (1, 1, 4, (3,)),
+])
+def test_flash_forward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype):
+    print("case b=%d nh=%d t=%d valid=%s dtype=%d" % (b, nh, t, valid, dtype), flush=True)
+    rng = np.random.default_rng(40)
+    q, k, v = (to16(rng.standard_normal((b, t, nh, HD)).astype(np.float32), tdtype) for _ in range(3))
+    o_ref, _, _ = reference_forward(q.float().numpy(), k.float().numpy(), v.float().numpy(), valid)
+    dq, dk, dv = q.cuda(), k.cuda(), v.cuda()
+    alibi = dev(orc.alibi(nh, t))
+    dvalid = dev(np.asarray(valid, np.int32))
+    o = torch.zeros((b, t, nh, HD), dtype=tdtype, device="cuda")
+    lse = empty((b, nh, t))
+    call("br_hip_flash_attn_fwd", ptr(dq), ptr(dk), ptr(dv), dtype, ptr(alibi), ptr(dvalid), ptr(o), ptr(lse), b, nh,
+         t, HD, nh * HD, HD, t * nh * HD, stream())
+    assert_close(host(o.float()), o_ref, TOL, "context")
+    # the same through [B, NH, T, HD] strides
+    zq, zk, zv = (x.permute(0, 2, 1, 3).contiguous() for x in (dq, dk, dv))
+    zo = torch.zeros((b, nh, t, HD), dtype=tdtype, device="cuda")
+    call("br_hip_flash_attn_fwd", ptr(zq), ptr(zk), ptr(zv), dtype, ptr(alibi), ptr(dvalid), ptr(zo), ptr(lse), b, nh,
+         t, HD, HD, t * HD, nh * t * HD, stream())
+    assert torch.equal(zo.permute(0, 2, 1, 3), o)
+    # log-sum-exp rows: exp(s - lse) must be the reference probabilities' normaliser
+    s = np.einsum("bqhd,bkhd->bhqk", q.float().numpy().astype(np.float64), k.float().numpy().astype(np.float64))
+    s = s / np.sqrt(HD) + orc.alibi(nh, t).astype(np.float64)[None, :, None, :]
+    vis = (np.arange(t)[None, :] <= np.arange(t)[:, None])[None] & (np.arange(t)[None, None, :] < np.asarray(valid)[:, None, None])
+    for bi in range(b):
+        if valid[bi] == 0:
+            continue
+        sm = np.where(vis[bi][None], s[bi], -np.inf)
+        want = np.log(np.exp(sm - sm.max(-1, keepdims=True)).sum(-1)) + sm.max(-1)
+        assert np.allclose(host(lse)[bi], want, rtol=0, atol=2e-2)
+
+
+def test_flash_forward_declines_unsupported_shapes():
+    lib = hip.load()
+    t = torch.zeros(4096, dtype=torch.float16, device="cuda")
+    f = empty(4096)
+    i = torch.ones(4, dtype=torch.int32, device="cuda")
+    ok = (ptr(t), ptr(t), ptr(t), F16, ptr(f), ptr(i), ptr(t), ptr(f))
+    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 8, 64, 64, 64, 512, stream()) == -1      # head size 64
+    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 6, 128, 128, 128, 768, stream()) == -1   # tokens % 4
+    assert lib.br_hip_flash_attn_fwd(ptr(t), ptr(t), ptr(t), hip.F32, ptr(f), ptr(i), ptr(t), ptr(f), 1, 1, 8, 128,
+                                     128, 128, 1024, stream()) == -1
+    assert lib.br_hip_flash_attn_fwd(None, ptr(t), ptr(t), F16, ptr(f), ptr(i), ptr(t), ptr(f), 1, 1, 8, 128, 128,
+                                     128, 1024, stream()) == -2
+    torch.cuda.synchronize()
