@@ -65,7 +65,7 @@ struct FlashArgs {
     float* lse;            // [batch, heads, tokens]
     float* delta;          // [batch, heads, tokens]  rowsum(dO o O)
     long long row, head, batch_stride;  // element strides of q, k, v, o, d_o, dq, dk, dv
-    int heads, tokens;
+    int heads, tokens, batch_heads;
     float scale;
 };
 
@@ -145,22 +145,46 @@ __device__ __forceinline__ float score(float dot, float scale, float bias, int q
     return key < tokens ? x : -INFINITY;  // tile overhang: not a key at all
 }
 
+// One LDS stage of the key loop: a K tile, a V tile and the tile's ALiBi row.
+constexpr int kTileBytes = kBK * kHD * 2;
+constexpr int kStageBytes = 2 * kTileBytes + kBK * 4;
+
+// Register staging of one stage (global -> registers -> LDS), so that the
+// loads of tile t+1 are in flight while tile t is computed.
+struct StageLoader {
+    TileLoader<kBK> k, v;
+    float bias;
+    __device__ __forceinline__ void fetch(const u16* kbase, const u16* vbase, const float* alibi_row, long long row,
+                                          int k0, int tokens) {
+        k.fetch(kbase, row, k0, tokens);
+        v.fetch(vbase, row, k0, tokens);
+        if (threadIdx.x < kBK) {
+            const int key = k0 + (int)threadIdx.x;
+            bias = alibi_row[key < tokens ? key : tokens - 1];
+        }
+    }
+    __device__ __forceinline__ void store(unsigned char* stage) const {
+        k.store(stage);
+        v.store(stage + kTileBytes);
+        if (threadIdx.x < kBK) reinterpret_cast<float*>(stage + 2 * kTileBytes)[threadIdx.x] = bias;
+    }
+};
+
 template <int CT>
-__global__ __launch_bounds__(kThreads) void flash_fwd_kernel(FlashArgs a) {
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_k[kBK * kHD * 2];
-    __shared__ __attribute__((aligned(1024))) unsigned char lds_v[kBK * kHD * 2];
-    const lds_byte* tk = (const lds_byte*)lds_k;
-    const lds_byte* tv = (const lds_byte*)lds_v;
+__global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+    // workgroups are numbered longest first: the query tiles with the most
+    // visible keys of every (batch, head), then the next ones, ...
     const int tiles_q = (a.tokens + kBQ - 1) / kBQ;
-    const int qt = tiles_q - 1 - (int)blockIdx.x;  // longest rows first
-    const int bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
+    const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
+    const int qt = tiles_q - 1 - (int)(blockIdx.x / a.batch_heads);
     const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
-    const int valid = a.valid[b];
+    const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
     const int q0 = qt * kBQ + wave * 32;
     const int query = q0 + (lane & 31);
     const int qrow = query < a.tokens ? query : a.tokens - 1;
-    const float* bias = a.alibi + (long long)h * a.tokens;
+    const float* alibi_row = a.alibi + (long long)h * a.tokens;
 
     u32x4 qf[8];
 #pragma unroll
@@ -179,75 +203,89 @@ __global__ __launch_bounds__(kThreads) void flash_fwd_kernel(FlashArgs a) {
     // keys this wave's queries can see (a wave may idle through the last tiles)
     const int wave_keys = visible_keys(q0 + 32, valid, a.tokens);
 
-    TileLoader<kBK> lk, lv;
-    lk.fetch(a.k + base, a.row, 0, a.tokens);
-    lv.fetch(a.v + base, a.row, 0, a.tokens);
+    StageLoader ld;
+    ld.fetch(a.k + base, a.v + base, alibi_row, a.row, 0, a.tokens);
+    ld.store(lds);
+    if (ntiles > 1) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, kBK, a.tokens);
+    __syncthreads();
     for (int t = 0; t < ntiles; t++) {
         const int k0 = t * kBK;
-        __syncthreads();  // every wave has finished reading the previous tile
-        lk.store(lds_k);
-        lv.store(lds_v);
-        __syncthreads();
-        if (t + 1 < ntiles) {
-            lk.fetch(a.k + base, a.row, k0 + kBK, a.tokens);
-            lv.fetch(a.v + base, a.row, k0 + kBK, a.tokens);
-        }
-        if (k0 >= wave_keys) continue;
-
-        f32x16 s[2];
+        const unsigned char* stage = lds + (t & 1) * kStageBytes;
+        const lds_byte* tk = (const lds_byte*)stage;
+        const lds_byte* tv = (const lds_byte*)(stage + kTileBytes);
+        const float* tb = reinterpret_cast<const float*>(stage + 2 * kTileBytes);
+        if (k0 < wave_keys) {
+            f32x16 s[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) s[kb][v] = 0.f;
+                for (int v = 0; v < 16; v++) s[kb][v] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 8; ks++) s[kb] = Cvt<CT>::mfma(frag_rows(tk, kb * 32, ks, lane), qf[ks], s[kb]);
-        }
-        float mt = -INFINITY;
+                for (int ks = 0; ks < 8; ks++)
+                    s[kb] = Cvt<CT>::mfma(frag_rows(tk, kb * 32, ks, lane), qf[ks], s[kb]);
+            }
+            // tiles wholly below the diagonal and inside the sequence need no mask
+            const bool open = k0 + kBK - 1 <= q0 && k0 + kBK <= valid;
+            float mt = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int key = k0 + kb * 32 + g * 8 + half * 4;
-                const int kidx = key + 3 < a.tokens ? key : a.tokens - 4;  // keep the 16-byte read inside the table
-                const float4 bv = *reinterpret_cast<const float4*>(bias + (kidx > 0 ? kidx : 0));
-                const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+                for (int g = 0; g < 4; g++) {
+                    const int kk = kb * 32 + g * 8 + half * 4;
+                    const float4 bv = *reinterpret_cast<const float4*>(tb + kk);
+                    const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const float x = score(s[kb][g * 4 + j], a.scale, bb[j], query, key + j, valid, a.tokens);
-                    s[kb][g * 4 + j] = x;
-                    mt = fmaxf(mt, x);
+                    for (int j = 0; j < 4; j++) {
+                        float x;
+                        if (open) {
+                            x = s[kb][g * 4 + j] * a.scale;
+                            x += bb[j];
+                        } else {
+                            x = score(s[kb][g * 4 + j], a.scale, bb[j], query, k0 + kk + j, valid, a.tokens);
+                        }
+                        s[kb][g * 4 + j] = x;
+                        mt = fmaxf(mt, x);
+                    }
                 }
+            mt = fmaxf(mt, xor32(mt));
+            const float m_new = fmaxf(m, mt);
+            const float alpha = __expf(m - m_new);
+            float sum = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float p = __expf(s[kb][v] - m_new);
+                    s[kb][v] = p;
+                    sum += p;
+                }
+            sum += xor32(sum);
+            l = l * alpha + sum;
+            m = m_new;
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) o[db][v] *= alpha;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int kb = j >> 1, vb = (j & 1) * 8;
+                float p8[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) p8[e] = s[kb][vb + e];
+                const u32x4 pf = pack8<CT>(p8);
+                const int ra = kb * 32 + (j & 1) * 16 + half * 4;
+#pragma unroll
+                for (int db = 0; db < 4; db++)
+                    o[db] = Cvt<CT>::mfma(frag_cols(tv, db * 32, ra, ra + 8, lane), pf, o[db]);
             }
-        mt = fmaxf(mt, xor32(mt));
-        const float m_new = fmaxf(m, mt);
-        const float alpha = __expf(m - m_new);
-        float sum = 0.f;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float p = __expf(s[kb][v] - m_new);
-                s[kb][v] = p;
-                sum += p;
-            }
-        sum += xor32(sum);
-        l = l * alpha + sum;
-        m = m_new;
-#pragma unroll
-        for (int db = 0; db < 4; db++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) o[db][v] *= alpha;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int kb = j >> 1, vb = (j & 1) * 8;
-            float p8[8];
-#pragma unroll
-            for (int e = 0; e < 8; e++) p8[e] = s[kb][vb + e];
-            const u32x4 pf = pack8<CT>(p8);
-            const int ra = kb * 32 + (j & 1) * 16 + half * 4;
-#pragma unroll
-            for (int db = 0; db < 4; db++) o[db] = Cvt<CT>::mfma(frag_cols(tv, db * 32, ra, ra + 8, lane), pf, o[db]);
         }
+        // tile t+1 (in registers since the previous iteration) goes into the
+        // other stage, whose last readers passed the barrier of iteration t-1
+        if (t + 1 < ntiles) {
+            ld.store(lds + ((t + 1) & 1) * kStageBytes);
+            if (t + 2 < ntiles) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, k0 + 2 * kBK, a.tokens);
+        }
+        __syncthreads();
     }
 
     if (query < a.tokens) {
@@ -266,10 +304,309 @@ __global__ __launch_bounds__(kThreads) void flash_fwd_kernel(FlashArgs a) {
     }
 }
 
+// ------------------------------------------------------------------ backward
+template <int CT>
+__device__ __forceinline__ float to_f32(u16 x);
+template <>
+__device__ __forceinline__ float to_f32<BR_GEMM_F16>(u16 x) { return (float)__builtin_bit_cast(_Float16, x); }
+template <>
+__device__ __forceinline__ float to_f32<BR_GEMM_BF16>(u16 x) { return __uint_as_float((unsigned)x << 16); }
+
+// delta[b, h, t] = sum_d dO[b, t, h, d] * O[b, t, h, d]: 16 lanes per row.
+template <int CT>
+__global__ __launch_bounds__(kThreads) void flash_delta_kernel(FlashArgs a, long long rows) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    long long r = idx >> 4;
+    const bool live = r < rows;
+    r = live ? r : rows - 1;
+    const int part = (int)(idx & 15);
+    const int h = (int)(r % a.heads);
+    const long long bt = r / a.heads;
+    const int t = (int)(bt % a.tokens);
+    const long long b = bt / a.tokens;
+    const long long off = b * a.batch_stride + (long long)t * a.row + (long long)h * a.head + part * 8;
+    const u32x4 g = *reinterpret_cast<const u32x4*>(a.d_o + off);
+    const u32x4 y = *reinterpret_cast<const u32x4*>(a.o + off);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        sum += to_f32<CT>((u16)(g[j] & 0xffffu)) * to_f32<CT>((u16)(y[j] & 0xffffu));
+        sum += to_f32<CT>((u16)(g[j] >> 16)) * to_f32<CT>((u16)(y[j] >> 16));
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
+    if (live && part == 0) a.delta[(b * a.heads + h) * a.tokens + t] = sum;
+}
+
+// One LDS stage of the query loop of the dK / dV pass: a Q tile, a dO tile and
+// the tile's lse and delta values.
+constexpr int kQStageBytes = 2 * kTileBytes + 2 * kBK * 4;
+
+struct QStageLoader {
+    TileLoader<kBK> q, g;
+    float stat;
+    __device__ __forceinline__ void fetch(const FlashArgs& a, long long base, int bh, int q0) {
+        q.fetch(a.q + base, a.row, q0, a.tokens);
+        g.fetch(a.d_o + base, a.row, q0, a.tokens);
+        if (threadIdx.x < 2 * kBK) {
+            const int t = q0 + (int)(threadIdx.x & (kBK - 1));
+            const float* src = threadIdx.x < kBK ? a.lse : a.delta;
+            stat = src[(long long)bh * a.tokens + (t < a.tokens ? t : a.tokens - 1)];
+        }
+    }
+    __device__ __forceinline__ void store(unsigned char* stage) const {
+        q.store(stage);
+        g.store(stage + kTileBytes);
+        if (threadIdx.x < 2 * kBK) reinterpret_cast<float*>(stage + 2 * kTileBytes)[threadIdx.x] = stat;
+    }
+};
+
+// dK, dV of 128 keys (32 per wave) of one (batch, head): queries stream through
+// LDS in tiles of 64.  Per wave and 32-query block:
+//   S[query, key]  = Q . K^T        (A = Q rows from LDS, B = K in registers)
+//   dP[query, key] = dO . V^T       (A = dO rows from LDS, B = V in registers)
+//   P = exp(score - lse),  dS = P o (dP - delta)
+//   dV[key, d] += P^T . dO,  dK[key, d] += dS^T . Q   (A from the accumulators,
+//                                    B by transposing reads of the same tiles)
+template <int CT>
+__global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kQStageBytes];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+    const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
+    const int kt = (int)(blockIdx.x / a.batch_heads);  // key tile 0 meets the most queries: longest first
+    const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
+    const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
+    const int key0 = kt * kBQ + wave * 32;
+    const int key = key0 + (lane & 31);
+    const int krow = key < a.tokens ? key : a.tokens - 1;
+    const float bias = a.alibi[(long long)h * a.tokens + krow];
+    const float uniform = 1.0f / (float)a.tokens;
+
+    u32x4 kf[8], vf[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+        kf[ks] = *reinterpret_cast<const u32x4*>(a.k + base + (long long)krow * a.row + ks * 16 + half * 8);
+        vf[ks] = *reinterpret_cast<const u32x4*>(a.v + base + (long long)krow * a.row + ks * 16 + half * 8);
+    }
+    f32x16 dk[4], dv[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) dk[db][v] = dv[db][v] = 0.f;
+
+    // queries that can see any key of this workgroup start at its first key
+    // (none at all when the keys lie in the padding); an empty sequence has
+    // uniform probabilities everywhere, so nothing is skipped for it
+    const bool dead_group = valid > 0 && kt * kBQ >= valid;
+    const int q_begin = valid > 0 ? (kt * kBQ / kBK) * kBK : 0;
+    const int ntiles = dead_group ? 0 : (a.tokens - q_begin + kBK - 1) / kBK;
+    const bool dead_wave = valid > 0 && key0 >= valid;
+
+    QStageLoader ld;
+    if (ntiles > 0) {
+        ld.fetch(a, base, bh, q_begin);
+        ld.store(lds);
+        if (ntiles > 1) ld.fetch(a, base, bh, q_begin + kBK);
+    }
+    __syncthreads();
+    for (int t = 0; t < ntiles; t++) {
+        const int q0 = q_begin + t * kBK;
+        const unsigned char* stage = lds + (t & 1) * kQStageBytes;
+        const lds_byte* tq = (const lds_byte*)stage;
+        const lds_byte* tg = (const lds_byte*)(stage + kTileBytes);
+        const float* tl = reinterpret_cast<const float*>(stage + 2 * kTileBytes);
+        const float* td = tl + kBK;
+        // a tile whose queries all precede this wave's keys sees none of them
+        if (!dead_wave && !(valid > 0 && q0 + kBK - 1 < key0)) {
+            const bool open = q0 >= key0 + 31 && key0 + 32 <= valid && q0 + kBK <= a.tokens;
+#pragma unroll
+            for (int qb = 0; qb < 2; qb++) {
+                f32x16 s, dp;
+#pragma unroll
+                for (int v = 0; v < 16; v++) s[v] = dp[v] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 8; ks++) {
+                    s = Cvt<CT>::mfma(frag_rows(tq, qb * 32, ks, lane), kf[ks], s);
+                    dp = Cvt<CT>::mfma(frag_rows(tg, qb * 32, ks, lane), vf[ks], dp);
+                }
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int qq = qb * 32 + g * 8 + half * 4;
+                    const float4 l4 = *reinterpret_cast<const float4*>(tl + qq);
+                    const float4 d4 = *reinterpret_cast<const float4*>(td + qq);
+                    const float ll[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int query = q0 + qq + j;
+                        float p;
+                        if (open) {
+                            float x = s[g * 4 + j] * a.scale;
+                            x += bias;
+                            p = __expf(x - ll[j]);
+                        } else {
+                            const float x = score(s[g * 4 + j], a.scale, bias, query, key, valid, a.tokens);
+                            p = valid > 0 ? __expf(x - ll[j]) : uniform;
+                            p = (query < a.tokens && key < a.tokens) ? p : 0.f;
+                        }
+                        s[g * 4 + j] = p;
+                        dp[g * 4 + j] = p * (dp[g * 4 + j] - dd[j]);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    float p8[8], s8[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        p8[e] = s[j * 8 + e];
+                        s8[e] = dp[j * 8 + e];
+                    }
+                    const u32x4 pf = pack8<CT>(p8), sf = pack8<CT>(s8);
+                    const int ra = qb * 32 + j * 16 + half * 4;
+#pragma unroll
+                    for (int db = 0; db < 4; db++) {
+                        dv[db] = Cvt<CT>::mfma(pf, frag_cols(tg, db * 32, ra, ra + 8, lane), dv[db]);
+                        dk[db] = Cvt<CT>::mfma(sf, frag_cols(tq, db * 32, ra, ra + 8, lane), dk[db]);
+                    }
+                }
+            }
+        }
+        if (t + 1 < ntiles) {
+            ld.store(lds + ((t + 1) & 1) * kQStageBytes);
+            if (t + 2 < ntiles) ld.fetch(a, base, bh, q0 + 2 * kBK);
+        }
+        __syncthreads();
+    }
+
+    // accumulator element v of block db: key key0 + acc_row(v), d = 32 * db + lane % 32
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        const int kk = key0 + acc_row(v, lane);
+        if (kk < a.tokens) {
+            const long long off = base + (long long)kk * a.row + (lane & 31);
+#pragma unroll
+            for (int db = 0; db < 4; db++) {
+                a.dk[off + db * 32] = dk[db][v] * a.scale;
+                a.dv[off + db * 32] = dv[db][v];
+            }
+        }
+    }
+}
+
+// dQ of 128 queries (32 per wave) of one (batch, head): the forward's loop over
+// key tiles, with  S^T = K . Q^T,  dP^T = V . dO^T  and
+// dQ^T[d, query] += K^T . dS^T  (K^T by transposing reads of the K tile).
+template <int CT>
+__global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+    const int tiles_q = (a.tokens + kBQ - 1) / kBQ;
+    const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
+    const int qt = tiles_q - 1 - (int)(blockIdx.x / a.batch_heads);
+    const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
+    const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
+    const int q0 = qt * kBQ + wave * 32;
+    const int query = q0 + (lane & 31);
+    const int qrow = query < a.tokens ? query : a.tokens - 1;
+    const float* alibi_row = a.alibi + (long long)h * a.tokens;
+    const float lse = a.lse[(long long)bh * a.tokens + qrow];
+    const float delta = a.delta[(long long)bh * a.tokens + qrow];
+    const float uniform = 1.0f / (float)a.tokens;
+
+    u32x4 qf[8], gf[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+        qf[ks] = *reinterpret_cast<const u32x4*>(a.q + base + (long long)qrow * a.row + ks * 16 + half * 8);
+        gf[ks] = *reinterpret_cast<const u32x4*>(a.d_o + base + (long long)qrow * a.row + ks * 16 + half * 8);
+    }
+    f32x16 dq[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) dq[db][v] = 0.f;
+
+    const int nkeys = visible_keys(qt * kBQ + kBQ, valid, a.tokens);
+    const int ntiles = (nkeys + kBK - 1) / kBK;
+    const int wave_keys = visible_keys(q0 + 32, valid, a.tokens);
+
+    StageLoader ld;
+    ld.fetch(a.k + base, a.v + base, alibi_row, a.row, 0, a.tokens);
+    ld.store(lds);
+    if (ntiles > 1) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, kBK, a.tokens);
+    __syncthreads();
+    for (int t = 0; t < ntiles; t++) {
+        const int k0 = t * kBK;
+        const unsigned char* stage = lds + (t & 1) * kStageBytes;
+        const lds_byte* tk = (const lds_byte*)stage;
+        const lds_byte* tv = (const lds_byte*)(stage + kTileBytes);
+        const float* tb = reinterpret_cast<const float*>(stage + 2 * kTileBytes);
+        if (k0 < wave_keys) {
+            const bool open = k0 + kBK - 1 <= q0 && k0 + kBK <= valid;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                f32x16 s, dp;
+#pragma unroll
+                for (int v = 0; v < 16; v++) s[v] = dp[v] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 8; ks++) {
+                    s = Cvt<CT>::mfma(frag_rows(tk, kb * 32, ks, lane), qf[ks], s);
+                    dp = Cvt<CT>::mfma(frag_rows(tv, kb * 32, ks, lane), gf[ks], dp);
+                }
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int kk = kb * 32 + g * 8 + half * 4;
+                    const float4 bv = *reinterpret_cast<const float4*>(tb + kk);
+                    const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float p;
+                        if (open) {
+                            float x = s[g * 4 + j] * a.scale;
+                            x += bb[j];
+                            p = __expf(x - lse);
+                        } else {
+                            const float x = score(s[g * 4 + j], a.scale, bb[j], query, k0 + kk + j, valid, a.tokens);
+                            p = valid > 0 ? __expf(x - lse) : uniform;
+                            p = k0 + kk + j < a.tokens ? p : 0.f;
+                        }
+                        dp[g * 4 + j] = p * (dp[g * 4 + j] - delta);
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    float s8[8];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) s8[e] = dp[j * 8 + e];
+                    const u32x4 sf = pack8<CT>(s8);
+                    const int ra = kb * 32 + j * 16 + half * 4;
+#pragma unroll
+                    for (int db = 0; db < 4; db++)
+                        dq[db] = Cvt<CT>::mfma(frag_cols(tk, db * 32, ra, ra + 8, lane), sf, dq[db]);
+                }
+            }
+        }
+        if (t + 1 < ntiles) {
+            ld.store(lds + ((t + 1) & 1) * kStageBytes);
+            if (t + 2 < ntiles) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, k0 + 2 * kBK, a.tokens);
+        }
+        __syncthreads();
+    }
+
+    if (query < a.tokens) {
+        float* row = a.dq + base + (long long)query * a.row;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                *reinterpret_cast<float4*>(row + db * 32 + g * 8 + half * 4) =
+                    make_float4(dq[db][g * 4 + 0] * a.scale, dq[db][g * 4 + 1] * a.scale, dq[db][g * 4 + 2] * a.scale,
+                                dq[db][g * 4 + 3] * a.scale);
+    }
+}
+
 bool flash_shape_ok(int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim, int64_t row, int64_t head,
                     int64_t batch_stride) {
     return batch > 0 && heads > 0 && tokens >= 4 && tokens % 4 == 0 && head_dim == kHD && row % 8 == 0 &&
-           head % 8 == 0 && batch_stride % 8 == 0 && batch * heads <= 65535 && tokens <= (1 << 20);
+           head % 8 == 0 && batch_stride % 8 == 0 && batch * heads <= (1 << 20) && tokens <= (1 << 20);
 }
 
 }  // namespace
@@ -301,12 +638,63 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
     a.batch_stride = batch_stride;
     a.heads = (int)heads;
     a.tokens = (int)tokens;
+    a.batch_heads = (int)(batch * heads);
     a.scale = (float)(1.0 / sqrt((double)head_dim));
-    const dim3 grid((unsigned)((tokens + kBQ - 1) / kBQ), (unsigned)(batch * heads));
+    const unsigned grid = (unsigned)(((tokens + kBQ - 1) / kBQ) * batch * heads);
     if (dtype == BR_F16)
         flash_fwd_kernel<BR_GEMM_F16><<<grid, kThreads, 0, as_stream(stream)>>>(a);
     else
         flash_fwd_kernel<BR_GEMM_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(a);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
+int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, int dtype,
+                          const float* alibi, const int32_t* valid, const float* lse, float* delta, float* dq,
+                          float* dk, float* dv, int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim,
+                          int64_t row_stride, int64_t head_stride, int64_t batch_stride, br_stream_t stream) {
+    if (batch < 0 || heads <= 0 || tokens <= 0 || head_dim <= 0) return BR_ERR_ATTR;
+    if (batch == 0) return BR_OK;
+    if (!q || !k || !v || !o || !d_o || !alibi || !valid || !lse) return BR_ERR_INPUT;
+    if (!delta || !dq || !dk || !dv) return BR_ERR_OUTPUT;
+    if ((dtype != BR_F16 && dtype != BR_BF16) ||
+        !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride) || !aligned16(q) ||
+        !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(alibi) || !aligned16(dq) ||
+        !aligned16(dk) || !aligned16(dv))
+        return BR_ERR_TODO;
+    FlashArgs a = {};
+    a.q = (const u16*)q;
+    a.k = (const u16*)k;
+    a.v = (const u16*)v;
+    a.o = (u16*)const_cast<void*>(o);
+    a.d_o = (const u16*)d_o;
+    a.dq = dq;
+    a.dk = dk;
+    a.dv = dv;
+    a.alibi = alibi;
+    a.valid = valid;
+    a.lse = const_cast<float*>(lse);
+    a.delta = delta;
+    a.row = row_stride;
+    a.head = head_stride;
+    a.batch_stride = batch_stride;
+    a.heads = (int)heads;
+    a.tokens = (int)tokens;
+    a.batch_heads = (int)(batch * heads);
+    a.scale = (float)(1.0 / sqrt((double)head_dim));
+    hipStream_t st = as_stream(stream);
+    const long long rows = batch * tokens * heads;
+    const unsigned tiles = (unsigned)(((tokens + kBQ - 1) / kBQ) * batch * heads);
+    const unsigned dgrid = (unsigned)((rows * 16 + kThreads - 1) / kThreads);
+    if (dtype == BR_F16) {
+        flash_delta_kernel<BR_GEMM_F16><<<dgrid, kThreads, 0, st>>>(a, rows);
+        flash_bwd_dkv_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
+        flash_bwd_dq_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
+    } else {
+        flash_delta_kernel<BR_GEMM_BF16><<<dgrid, kThreads, 0, st>>>(a, rows);
+        flash_bwd_dkv_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
+        flash_bwd_dq_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
+    }
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }

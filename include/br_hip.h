@@ -299,6 +299,21 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
                           int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
                           int64_t batch_stride, br_stream_t stream);
 
+/* Backward of br_hip_flash_attn_fwd: the chain op_attn_backward
+ * (cuda_tensor.cpp:830-888), op_softmax_backward (:890-918) and op_qk_backward
+ * (:1004-1063) of train.words:217-226 without the [batch, heads, tokens, tokens]
+ * tensors: probabilities are recomputed from q, k and lse.  o is the forward's
+ * output, d_o its gradient (both `dtype`, same strides as q, k, v); dq, dk, dv
+ * are fp32 with the same element strides.  delta: fp32 scratch of
+ * batch * heads * tokens entries (receives rowsum(d_o * o)).  Deterministic: one
+ * pass accumulates dk / dv per key block, a second one dq per query block.
+ * Same shape limits as the forward (BR_ERR_TODO otherwise). */
+int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
+                          int dtype, const float* alibi, const int32_t* valid, const float* lse,
+                          float* delta, float* dq, float* dk, float* dv, int64_t batch, int64_t heads,
+                          int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
+                          int64_t batch_stride, br_stream_t stream);
+
 /* ---- optimizer ---------------------------------------------------------- */
 /* One AdamW step (decoupled weight decay) over n parameters, all arithmetic in
  * fp32:  p *= 1 - lr*wd;  m += (g - m)(1 - beta1);  v = beta2 v + (1 - beta2) g^2;
