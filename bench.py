@@ -110,19 +110,29 @@ def block_leg(args, host, hip, timer):
     env.write("xinput", normal((B, T, H), 1.0))
     env.write("yout_g0", normal((B, T, H), 1.0))
     env.write("mask_", np.ones((B, T), np.int32))
-    env.execute("create_operand_buffers prepare_batch op.sync")
+    env.execute("create_operand_buffers create_flash_buffers prepare_batch_flash op.sync")
     # the backward adds into yout_g in place, so every step starts from a fresh copy.
-    # block_step_mixed = the same operator sequence with product-only operands kept in
-    # fp16 buffers; it produces the bits block_step produces (tests/test_gpu_block.py).
-    step = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step_mixed")
+    # block_step        the reference's operator sequence over the fp32 arena
+    # block_step_mixed  the same sequence with product-only operands kept in fp16 buffers;
+    #                   it produces the bits block_step produces (tests/test_gpu_block.py)
+    # block_step_flash  block_step_mixed with the attention chain as one fused kernel per
+    #                   direction (same tolerance against the oracle, not the same bits)
+    step = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step_flash")
+    mixed = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step_mixed")
     plain = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step")
     sec = timer.run(lambda i: env.run(step), args.steps, args.warmup)
+    out_flash = env.read("xa")
+    assert np.all(np.isfinite(out_flash)), "block step produced non-finite values"
+    few = max(3, args.steps // 4)
+    sec_mixed = timer.run(lambda i: env.run(mixed), few, 1)
     out = env.read("xa")
-    assert np.all(np.isfinite(out)), "block step produced non-finite values"
-    sec_plain = timer.run(lambda i: env.run(plain), max(3, args.steps // 4), 1)
-    assert np.array_equal(env.read("xa"), out), "the two word sets disagree"
+    sec_plain = timer.run(lambda i: env.run(plain), few, 1)
+    assert np.array_equal(env.read("xa"), out), "the two operator-chain word sets disagree"
+    scale = float(np.sqrt(np.mean(out.astype(np.float64) ** 2)))
+    assert float(np.max(np.abs(out_flash - out))) <= 2e-2 * (float(np.max(np.abs(out))) + scale), \
+        "fused attention and the operator chain disagree"
     env.close()
-    return sec, sec_plain
+    return sec, sec_mixed, sec_plain
 
 
 def model_leg(args, host, timer):
@@ -363,7 +373,8 @@ def main():
                                      "weights ~N(0,0.02), fp32 activations and accumulation, seed 3",
                          "tokens_per_step": N, "gemm_gflop_per_step": STEP_GEMM_FLOP / 1e9}}
     if args.leg in ("all", "block"):
-        sec, sec_plain = block_leg(args, host, hip, timer)
+        sec, sec_mixed, sec_plain = block_leg(args, host, hip, timer)
+        result["ms_per_step_operator_chain_fp16_buffers"] = sec_mixed * 1e3
         result["ms_per_step_fp32_arena_words"] = sec_plain * 1e3
         result["value"] = N / sec
         result["ms_per_step"] = sec * 1e3

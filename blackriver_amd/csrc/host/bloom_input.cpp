@@ -3,6 +3,7 @@
 #include <cfloat>
 #include <cmath>
 #include <cstring>
+#include <vector>
 
 #include "br_hip.h"
 #include "runtime.hpp"
@@ -114,6 +115,33 @@ struct XMask : public NativeWord {
     NWORD_CREATOR_DEFINE_LR(XMask)
 };
 
+// ( mask valid -- )  valid[b] = number of leading non-zero entries of mask[b, :]
+// (for a batch padded on the right: the sequence length), as int32 values in
+// the storage of a 4-byte-element device tensor; the fused attention words
+// derive the causal / padding mask from it instead of reading the mask table.
+struct Valid : public NativeWord {
+    void run(Stack& stack) override {
+        tensor_t valid = stack.pop_tensor();
+        tensor_t mask = stack.pop_tensor();
+        br_assert(mask->is_cpu() && mask->dtype() == DataType::Int && mask->shape().dim() == 2,
+                  "bloom.valid: mask must be a [batch, tokens] cpu int tensor");
+        const int64_t batch = (int64_t)mask->shape()[0], tokens = (int64_t)mask->shape()[1];
+        br_assert(valid->is_cuda() && valid->dtype() == DataType::Float && (int64_t)valid->items() >= batch,
+                  "bloom.valid: expects a device fp32-typed tensor of at least batch entries");
+        std::vector<int32_t> count((size_t)batch);
+        const int32_t* m = static_cast<const int32_t*>(mask->data());
+        for (int64_t b = 0; b < batch; b++) {
+            int64_t n = 0;
+            while (n < tokens && m[b * tokens + n] != 0) n++;
+            count[(size_t)b] = (int32_t)n;
+        }
+        BR_HIP_CHECK(br_hip_memcpy_h2d(valid->data(), count.data(), (size_t)batch * sizeof(int32_t),
+                                       ComputingContext::stream));
+        ComputingContext::sync();  // `count` leaves scope; once per batch
+    }
+    NWORD_CREATOR_DEFINE_LR(Valid)
+};
+
 // ( tensor mean std seed -- )  synthetic initialisation of a device tensor
 struct Normal : public NativeWord {
     void run(Stack& stack) override {
@@ -143,6 +171,7 @@ void load_bloom_words(Enviroment& env) {
     env.insert_native_word("bloom.embed_backward", EmbedBackward::creator);
     env.insert_native_word("bloom.alibi", Alibi::creator);
     env.insert_native_word("bloom.xmask", XMask::creator);
+    env.insert_native_word("bloom.valid", Valid::creator);
 }
 
 }  // namespace br

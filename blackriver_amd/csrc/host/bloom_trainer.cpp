@@ -30,6 +30,10 @@ bool BloomTrainer::mixed() const {
     return cfg_.weight_dtype == cfg_.gemm_precision && (cfg_.weight_dtype == "f16" || cfg_.weight_dtype == "bf16");
 }
 
+bool BloomTrainer::flash() const {
+    return cfg_.fused_attention && mixed() && cfg_.hidden / cfg_.heads == 128 && cfg_.tokens % 4 == 0;
+}
+
 int64_t BloomTrainer::model_arena_floats() const {
     // plus one logits row per position: the loss head then needs a single group
     return block_arena_floats() + cfg_.batch * cfg_.tokens * cfg_.vocab;
@@ -56,6 +60,7 @@ std::string BloomTrainer::setup_script() const {
         s << block_arena_floats() + cfg_.vocab << " create_var\n";
         s << cfg_.batch << " " << cfg_.tokens << " create_dynamic_here\n";
         if (mixed()) s << "create_operand_buffers\n";
+        if (flash()) s << "create_flash_buffers\n";
         s << "0 #  " << i << " share_batch_tensors\n";
     }
     s << "0 #\n";
@@ -65,8 +70,8 @@ std::string BloomTrainer::setup_script() const {
 std::string BloomTrainer::step_script() const {
     std::ostringstream s;
     const int n = cfg_.layers;
-    const char* forward = mixed() ? "layer_forward_mixed" : "layer_forward";
-    const char* backward = mixed() ? "layer_backward_mixed" : "layer_backward_core";
+    const char* forward = flash() ? "layer_forward_flash" : mixed() ? "layer_forward_mixed" : "layer_forward";
+    const char* backward = flash() ? "layer_backward_flash" : mixed() ? "layer_backward_mixed" : "layer_backward_core";
     s << "0 # model_input\n";
     s << "1 # 'xinput' @  0 # 'xinput' @  op.copy   1 # " << forward << "\n";
     for (int i = 2; i <= n; i++)

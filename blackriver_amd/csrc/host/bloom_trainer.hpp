@@ -23,6 +23,9 @@ struct BloomModelConfig {
     float eps = 1e-5f;
     std::string weight_dtype = "f16";     // "float", "f16" or "bf16": storage of the weight matrices
     std::string gemm_precision = "f16";   // MFMA type for products of fp32-stored operands
+    // one fused attention kernel per direction instead of the operator chain
+    // through [B, heads, T, T] tensors; used when the shape allows (see flash())
+    bool fused_attention = true;
 };
 
 class BloomTrainer {
@@ -52,6 +55,8 @@ public:
     int64_t block_arena_floats() const;
     int64_t model_arena_floats() const;
     bool mixed() const;
+    // fused attention is on and applies: 16-bit operand buffers, head size 128, tokens % 4 == 0
+    bool flash() const;
     std::string setup_script() const;
     std::string step_script() const;
 

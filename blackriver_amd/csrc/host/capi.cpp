@@ -19,6 +19,7 @@ struct br_env {
     std::unique_ptr<Enviroment> env;
     std::vector<std::unique_ptr<DaG>> programs;
     std::unique_ptr<BloomTrainer> trainer;
+    bool fused_attention = true;
 };
 
 namespace {
@@ -279,9 +280,14 @@ int br_bloom_model_create(br_env_t* e, int layers, int64_t batch, int64_t tokens
         cfg.eps = eps;
         cfg.weight_dtype = weight_dtype ? weight_dtype : "f16";
         cfg.gemm_precision = gemm_precision ? gemm_precision : "f16";
+        cfg.fused_attention = e->fused_attention;
         e->trainer.reset(new BloomTrainer(*e->env, cfg));
         e->trainer->create();
     });
+}
+
+int br_bloom_model_set_fused_attention(br_env_t* e, int on) {
+    return guarded([&]() { e->fused_attention = on != 0; });
 }
 
 int br_bloom_model_init(br_env_t* e, uint64_t seed, float std) {

@@ -4,6 +4,8 @@
 // (blackriver/nn.cpp:16-337) so the model scripts run unchanged.
 #include "words.hpp"
 
+#include <vector>
+
 #include "br_hip.h"
 #include "runtime.hpp"
 #include "tensor.hpp"
@@ -215,6 +217,75 @@ BR_WORD(SoftmaxAttnBackward, Tensors<5> a(stack); a[0]->op_softmax_attn_backward
 // ( dS q k q_g k_g -- )
 BR_WORD(QueryKeyBackward, Tensors<5> a(stack); a[0]->op_qk_backward(a[0], a[1], a[2], a[3], a[4]);)
 
+// Fused attention (no counterpart in the reference, which runs the chain
+// op.querykey, op.add, op.add, op.softmax, op.attn and its backward through
+// [B, heads, T, T] tensors).  q, k, v, o, dO are 16-bit device tensors laid out
+// [B, T, heads, 128] (the projections' own output, no 0213 transposes); only
+// q's shape is consulted.  `valid` comes from bloom.valid (sequences padded on
+// the right), `alibi` is the table bloom.alibi builds.
+struct FlashOperands {
+    int64_t batch, tokens, heads, head_dim;
+    const int32_t* valid;  // device, [batch]
+};
+// `valid` is the tensor bloom.valid fills: per sequence the number of leading
+// real tokens, int32 values kept in the storage of a 4-byte-element device tensor.
+FlashOperands flash_operands(const tensor_t& q, const tensor_t& valid, const tensor_t& alibi) {
+    br_assert(q->shape().dim() == 4, "fused attention: q must be [batch, tokens, heads, head size]");
+    FlashOperands f;
+    f.batch = (int64_t)q->shape()[0];
+    f.tokens = (int64_t)q->shape()[1];
+    f.heads = (int64_t)q->shape()[2];
+    f.head_dim = (int64_t)q->shape()[3];
+    br_assert(valid->is_cuda() && valid->dtype() == DataType::Float && (int64_t)valid->items() >= f.batch,
+              "fused attention: valid must be the device tensor bloom.valid fills");
+    br_assert(alibi->is_cuda() && alibi->dtype() == DataType::Float && (int64_t)alibi->items() == f.heads * f.tokens,
+              "fused attention: alibi must be the fp32 [heads, tokens] table");
+    f.valid = static_cast<const int32_t*>(valid->data());
+    return f;
+}
+bool flash_16(const tensor_t& t, const tensor_t& q) {
+    return t->is_cuda() && t->dtype() == q->dtype() && t->items() == q->items();
+}
+bool flash_f32(const tensor_t& t, size_t items) {
+    return t->is_cuda() && t->dtype() == DataType::Float && t->items() == items;
+}
+// ( q k v alibi valid o lse -- )
+BR_WORD(FlashAttn,
+    Tensors<7> a(stack);
+    const tensor_t& q = a[0];
+    br_assert(q->is_cuda() && (q->dtype() == DataType::F16 || q->dtype() == DataType::BF16),
+              "op.flash_attn: 16-bit device tensors");
+    const FlashOperands f = flash_operands(q, a[4], a[3]);
+    br_assert(flash_16(a[1], q) && flash_16(a[2], q) && flash_16(a[5], q), "op.flash_attn: k, v, o must match q");
+    br_assert(flash_f32(a[6], (size_t)(f.batch * f.heads * f.tokens)), "op.flash_attn: lse is fp32 [batch, heads, tokens]");
+    BR_HIP_CHECK(br_hip_flash_attn_fwd(q->data(), a[1]->data(), a[2]->data(), (int)q->dtype(),
+                                       static_cast<const float*>(a[3]->data()), f.valid, a[5]->data(),
+                                       static_cast<float*>(a[6]->data()), f.batch, f.heads, f.tokens, f.head_dim,
+                                       f.heads * f.head_dim, f.head_dim, f.tokens * f.heads * f.head_dim,
+                                       ComputingContext::stream));
+)
+// ( q k v o dO alibi valid lse dq dk dv -- )   dq, dk, dv: fp32, same layout
+BR_WORD(FlashAttnBackward,
+    Tensors<11> a(stack);
+    const tensor_t& q = a[0];
+    br_assert(q->is_cuda() && (q->dtype() == DataType::F16 || q->dtype() == DataType::BF16),
+              "op.flash_attn_backward: 16-bit device tensors");
+    const FlashOperands f = flash_operands(q, a[6], a[5]);
+    float* delta = static_cast<float*>(ComputingContext::scratch((size_t)(f.batch * f.heads * f.tokens) * sizeof(float)));
+    br_assert(flash_16(a[1], q) && flash_16(a[2], q) && flash_16(a[3], q) && flash_16(a[4], q),
+              "op.flash_attn_backward: k, v, o, dO must match q");
+    br_assert(flash_f32(a[7], (size_t)(f.batch * f.heads * f.tokens)), "op.flash_attn_backward: lse");
+    br_assert(flash_f32(a[8], q->items()) && flash_f32(a[9], q->items()) && flash_f32(a[10], q->items()),
+              "op.flash_attn_backward: dq, dk, dv are fp32 tensors of q's size");
+    BR_HIP_CHECK(br_hip_flash_attn_bwd(q->data(), a[1]->data(), a[2]->data(), a[3]->data(), a[4]->data(),
+                                       (int)q->dtype(), static_cast<const float*>(a[5]->data()), f.valid,
+                                       static_cast<const float*>(a[7]->data()), delta,
+                                       static_cast<float*>(a[8]->data()), static_cast<float*>(a[9]->data()),
+                                       static_cast<float*>(a[10]->data()), f.batch, f.heads, f.tokens, f.head_dim,
+                                       f.heads * f.head_dim, f.head_dim, f.tokens * f.heads * f.head_dim,
+                                       ComputingContext::stream));
+)
+
 // AdamW on one parameter tensor.  The reference stops at the gradients; these
 // two words are what a training loop runs after them.
 // ( param [master] grad m v lr beta1 beta2 eps weight_decay step -- )
@@ -299,6 +370,8 @@ void load_nn_words(Enviroment& env) {
         {"op.softmax_backward", SoftmaxBackward::creator},
         {"op.softmax_attn_backward", SoftmaxAttnBackward::creator},
         {"op.qk_backward", QueryKeyBackward::creator},
+        {"op.flash_attn", FlashAttn::creator},
+        {"op.flash_attn_backward", FlashAttnBackward::creator},
         {"op.adamw", AdamW::creator},
         {"op.adamw_master", AdamWMaster::creator},
     };

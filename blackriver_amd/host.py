@@ -53,6 +53,7 @@ SIGNATURES = {
     "br_env_tensor_read_i32": (_int, [_vp, _cp, _i32p, _i64]),
     "br_host_set_echo_loss": (_int, [_int]),
     "br_bloom_model_create": (_int, [_vp, _int, _i64, _i64, _i64, _i64, _i64, ctypes.c_float, _cp, _cp]),
+    "br_bloom_model_set_fused_attention": (_int, [_vp, _int]),
     "br_bloom_model_init": (_int, [_vp, ctypes.c_uint64, ctypes.c_float]),
     "br_bloom_model_step": (_int, [_vp, _i32p, _i32p, ctypes.POINTER(ctypes.c_float)]),
     "br_bloom_model_optimizer_create": (_int, [_vp] + [ctypes.c_float] * 5),
@@ -246,12 +247,13 @@ class BloomModel:
     hash i of `env`, embedding / final LayerNorm / LM head in hash 0."""
 
     def __init__(self, layers, batch, tokens, hidden=4096, heads=32, vocab=250880, eps=1e-5, weight_dtype="f16",
-                 gemm_precision="f16"):
+                 gemm_precision="f16", fused_attention=True):
         self.layers, self.batch, self.tokens = layers, batch, tokens
         self.hidden, self.heads, self.vocab, self.eps = hidden, heads, vocab, eps
         self.env = Env(layers + 1)
         self.env.execute(words_text("bloom.words"))
         self.env.execute(words_text("bloom_model.words"))
+        _check(load().br_bloom_model_set_fused_attention(self.env._h, 1 if fused_attention else 0), "model_attention")
         _check(load().br_bloom_model_create(self.env._h, layers, batch, tokens, hidden, heads, vocab, eps,
                                             weight_dtype.encode(), gemm_precision.encode()), "model_create")
 

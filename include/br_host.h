@@ -99,6 +99,11 @@ int br_env_tensor_read_i32(br_env_t* env, const char* name, int32_t* dst, int64_
 int br_bloom_model_create(br_env_t* env, int layers, int64_t batch, int64_t tokens, int64_t hidden,
                           int64_t heads, int64_t vocab, float eps, const char* weight_dtype,
                           const char* gemm_precision);
+/* Before br_bloom_model_create: whether attention runs as one fused kernel per
+ * direction (default; applies with 16-bit weights multiplied in their own
+ * type, head size 128 and tokens % 4 == 0) or as the reference's operator
+ * chain through [batch, heads, tokens, tokens] tensors. */
+int br_bloom_model_set_fused_attention(br_env_t* env, int on);
 int br_bloom_model_init(br_env_t* env, uint64_t seed, float std);
 int br_bloom_model_step(br_env_t* env, const int32_t* ids, const int32_t* mask, float* loss);
 /* AdamW over every parameter of the model (the reference's loop ends at the

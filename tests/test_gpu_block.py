@@ -281,3 +281,35 @@ def test_qkv_relayout_words_match_the_offline_converter(runtime, dtype):
         assert np.array_equal(env.read("w.back"), w) and np.array_equal(env.read("b.back"), b)
     finally:
         env.close()
+
+
+@pytest.mark.parametrize("mode,tol", [("f16", 2e-2), ("bf16", 6e-2)])
+def test_block_with_fused_attention_matches_oracle(runtime, mode, tol):
+    """layer_forward_flash / layer_backward_flash (attention as one fused kernel
+    per direction, head size 128) against the oracle's operator-by-operator
+    block, and against the operand-buffer words within the same bound."""
+    hidden, heads, batch, tokens = 512, 4, 2, 64
+    env, w, x, dy, mask, _ = setup_block(runtime, hidden, heads, batch, tokens, mode)
+    env.execute("create_operand_buffers create_flash_buffers prepare_batch_flash")
+    env.execute("block_step_flash op.sync")
+    saved = blk.layer_forward(w, x, orc.alibi(heads, tokens), orc.xmask(mask), heads, 1e-5)
+    dx_ref, g_ref = blk.layer_backward(w, saved, x, dy, heads, 1e-5)
+    assert_close(env.read("xa"), dx_ref, tol, "dx")
+    got = {n: env.read(n) for n in ["xa"] + [k for k in g_ref]}
+    for name, ref in g_ref.items():
+        if name.startswith("key.bias"):
+            continue
+        if name.startswith(("query.", "key.", "value.")):
+            continue          # thirds of query_key_value, compared below
+        assert_close(got[name], ref, tol, name)
+    qkv_w = np.concatenate([g_ref["query.weight_g"], g_ref["key.weight_g"], g_ref["value.weight_g"]])
+    assert_close(env.read("query_key_value.weight_g"), qkv_w, tol, "query_key_value.weight_g")
+    # the forward output, from a fresh forward pass
+    env.write("xinput", x)
+    env.execute("layer_forward_flash op.sync")
+    assert_close(env.read("xa"), saved["xa"], tol, "block output")
+    flash_out = env.read("xa")
+    env.write("xinput", x)
+    env.execute("layer_forward_mixed op.sync")
+    assert_close(flash_out, env.read("xa"), tol, "flash vs operator chain")
+    env.close()

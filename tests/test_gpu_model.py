@@ -49,6 +49,7 @@ def build(mode, layers, batch, tokens, hidden, heads, vocab, seed):
 @pytest.mark.parametrize("mode,layers,batch,tokens,hidden,heads,vocab", [
     ("fp32", 3, 2, 32, 256, 4, 1024),
     ("f16", 2, 2, 64, 512, 8, 2048),
+    ("f16", 2, 2, 64, 512, 4, 2048),      # head size 128: attention runs as the fused kernels
 ])
 def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden, heads, vocab):
     print("case %s layers=%d batch=%d tokens=%d hidden=%d" % (mode, layers, batch, tokens, hidden), flush=True)
