@@ -262,7 +262,7 @@ BR_WORD(FlashAttn,
                                        static_cast<const float*>(a[3]->data()), f.valid, a[5]->data(),
                                        static_cast<float*>(a[6]->data()), f.batch, f.heads, f.tokens, f.head_dim,
                                        f.heads * f.head_dim, f.head_dim, f.tokens * f.heads * f.head_dim,
-                                       ComputingContext::stream));
+                                       f.heads * f.head_dim, f.tokens * f.heads * f.head_dim, ComputingContext::stream));
 )
 // ( q k v o dO alibi valid lse dq dk dv -- )   dq, dk, dv: fp32, same layout
 BR_WORD(FlashAttnBackward,
@@ -283,7 +283,49 @@ BR_WORD(FlashAttnBackward,
                                        static_cast<float*>(a[8]->data()), static_cast<float*>(a[9]->data()),
                                        static_cast<float*>(a[10]->data()), f.batch, f.heads, f.tokens, f.head_dim,
                                        f.heads * f.head_dim, f.head_dim, f.tokens * f.heads * f.head_dim,
+                                       f.heads * f.head_dim, f.tokens * f.heads * f.head_dim, ComputingContext::stream));
+)
+// The same on a packed projection: qkv is the [B, T, 3 * hidden] output of ONE
+// linear layer over the fused query_key_value weight (rows ordered q | k | v,
+// each [heads, 128]); o is [B, T, heads, 128] and its shape is the one consulted.
+// ( qkv alibi valid o lse -- )
+BR_WORD(FlashAttnQkv,
+    Tensors<5> a(stack);
+    const tensor_t& o = a[3];
+    br_assert(o->is_cuda() && (o->dtype() == DataType::F16 || o->dtype() == DataType::BF16),
+              "op.flash_attn_qkv: 16-bit device tensors");
+    const FlashOperands f = flash_operands(o, a[2], a[1]);
+    const int64_t hidden = f.heads * f.head_dim;
+    br_assert(a[0]->is_cuda() && a[0]->dtype() == o->dtype() && a[0]->items() == 3 * o->items(),
+              "op.flash_attn_qkv: qkv must hold three tensors of o's size and type");
+    br_assert(flash_f32(a[4], (size_t)(f.batch * f.heads * f.tokens)), "op.flash_attn_qkv: lse is fp32 [batch, heads, tokens]");
+    const char* qkv = static_cast<const char*>(a[0]->data());
+    BR_HIP_CHECK(br_hip_flash_attn_fwd(qkv, qkv + 2 * hidden, qkv + 4 * hidden, (int)o->dtype(),
+                                       static_cast<const float*>(a[1]->data()), f.valid, o->data(),
+                                       static_cast<float*>(a[4]->data()), f.batch, f.heads, f.tokens, f.head_dim,
+                                       3 * hidden, f.head_dim, f.tokens * 3 * hidden, hidden, f.tokens * hidden,
                                        ComputingContext::stream));
+)
+// ( qkv o dO alibi valid lse dqkv -- )   dqkv: fp32 [B, T, 3 * hidden], packed like qkv
+BR_WORD(FlashAttnQkvBackward,
+    Tensors<7> a(stack);
+    const tensor_t& o = a[1];
+    br_assert(o->is_cuda() && (o->dtype() == DataType::F16 || o->dtype() == DataType::BF16),
+              "op.flash_attn_qkv_backward: 16-bit device tensors");
+    const FlashOperands f = flash_operands(o, a[4], a[3]);
+    const int64_t hidden = f.heads * f.head_dim;
+    br_assert(a[0]->is_cuda() && a[0]->dtype() == o->dtype() && a[0]->items() == 3 * o->items() && flash_16(a[2], o),
+              "op.flash_attn_qkv_backward: qkv holds three tensors of o's size and type, dO matches o");
+    br_assert(flash_f32(a[5], (size_t)(f.batch * f.heads * f.tokens)), "op.flash_attn_qkv_backward: lse");
+    br_assert(flash_f32(a[6], 3 * o->items()), "op.flash_attn_qkv_backward: dqkv is fp32 of qkv's size");
+    float* delta = static_cast<float*>(ComputingContext::scratch((size_t)(f.batch * f.heads * f.tokens) * sizeof(float)));
+    const char* qkv = static_cast<const char*>(a[0]->data());
+    float* g = static_cast<float*>(a[6]->data());
+    BR_HIP_CHECK(br_hip_flash_attn_bwd(qkv, qkv + 2 * hidden, qkv + 4 * hidden, o->data(), a[2]->data(), (int)o->dtype(),
+                                       static_cast<const float*>(a[3]->data()), f.valid,
+                                       static_cast<const float*>(a[5]->data()), delta, g, g + hidden, g + 2 * hidden,
+                                       f.batch, f.heads, f.tokens, f.head_dim, 3 * hidden, f.head_dim,
+                                       f.tokens * 3 * hidden, hidden, f.tokens * hidden, ComputingContext::stream));
 )
 
 // AdamW on one parameter tensor.  The reference stops at the gradients; these
@@ -372,6 +414,8 @@ void load_nn_words(Enviroment& env) {
         {"op.qk_backward", QueryKeyBackward::creator},
         {"op.flash_attn", FlashAttn::creator},
         {"op.flash_attn_backward", FlashAttnBackward::creator},
+        {"op.flash_attn_qkv", FlashAttnQkv::creator},
+        {"op.flash_attn_qkv_backward", FlashAttnQkvBackward::creator},
         {"op.adamw", AdamW::creator},
         {"op.adamw_master", AdamWMaster::creator},
     };

@@ -64,7 +64,8 @@ struct FlashArgs {
     const int32_t* valid;  // [batch]
     float* lse;            // [batch, heads, tokens]
     float* delta;          // [batch, heads, tokens]  rowsum(dO o O)
-    long long row, head, batch_stride;  // element strides of q, k, v, o, d_o, dq, dk, dv
+    long long row, head, batch_stride;  // element strides of q, k, v, dq, dk, dv
+    long long orow, obatch;             // token / batch strides of o and d_o (same head stride)
     int heads, tokens, batch_heads;
     float scale;
 };
@@ -290,7 +291,7 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
 
     if (query < a.tokens) {
         const float inv = 1.0f / l;
-        u16* orow = a.o + base + (long long)query * a.row;
+        u16* orow = a.o + (long long)b * a.obatch + (long long)h * a.head + (long long)query * a.orow;
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(kThreads) void flash_delta_kernel(FlashArgs a, long
     const long long bt = r / a.heads;
     const int t = (int)(bt % a.tokens);
     const long long b = bt / a.tokens;
-    const long long off = b * a.batch_stride + (long long)t * a.row + (long long)h * a.head + part * 8;
+    const long long off = b * a.obatch + (long long)t * a.orow + (long long)h * a.head + part * 8;
     const u32x4 g = *reinterpret_cast<const u32x4*>(a.d_o + off);
     const u32x4 y = *reinterpret_cast<const u32x4*>(a.o + off);
     float sum = 0.f;
@@ -345,9 +346,9 @@ constexpr int kQStageBytes = 2 * kTileBytes + 2 * kBK * 4;
 struct QStageLoader {
     TileLoader<kBK> q, g;
     float stat;
-    __device__ __forceinline__ void fetch(const FlashArgs& a, long long base, int bh, int q0) {
+    __device__ __forceinline__ void fetch(const FlashArgs& a, long long base, long long obase, int bh, int q0) {
         q.fetch(a.q + base, a.row, q0, a.tokens);
-        g.fetch(a.d_o + base, a.row, q0, a.tokens);
+        g.fetch(a.d_o + obase, a.orow, q0, a.tokens);
         if (threadIdx.x < 2 * kBK) {
             const int t = q0 + (int)(threadIdx.x & (kBK - 1));
             const float* src = threadIdx.x < kBK ? a.lse : a.delta;
@@ -375,6 +376,7 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
     const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
     const int kt = (int)(blockIdx.x / a.batch_heads);  // key tile 0 meets the most queries: longest first
     const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
+    const long long obase = (long long)b * a.obatch + (long long)h * a.head;
     const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
     const int key0 = kt * kBQ + wave * 32;
     const int key = key0 + (lane & 31);
@@ -404,9 +406,9 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
 
     QStageLoader ld;
     if (ntiles > 0) {
-        ld.fetch(a, base, bh, q_begin);
+        ld.fetch(a, base, obase, bh, q_begin);
         ld.store(lds);
-        if (ntiles > 1) ld.fetch(a, base, bh, q_begin + kBK);
+        if (ntiles > 1) ld.fetch(a, base, obase, bh, q_begin + kBK);
     }
     __syncthreads();
     for (int t = 0; t < ntiles; t++) {
@@ -472,7 +474,7 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
         }
         if (t + 1 < ntiles) {
             ld.store(lds + ((t + 1) & 1) * kQStageBytes);
-            if (t + 2 < ntiles) ld.fetch(a, base, bh, q0 + 2 * kBK);
+            if (t + 2 < ntiles) ld.fetch(a, base, obase, bh, q0 + 2 * kBK);
         }
         __syncthreads();
     }
@@ -516,7 +518,8 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) {
         qf[ks] = *reinterpret_cast<const u32x4*>(a.q + base + (long long)qrow * a.row + ks * 16 + half * 8);
-        gf[ks] = *reinterpret_cast<const u32x4*>(a.d_o + base + (long long)qrow * a.row + ks * 16 + half * 8);
+        gf[ks] = *reinterpret_cast<const u32x4*>(a.d_o + (long long)b * a.obatch + (long long)h * a.head +
+                                                 (long long)qrow * a.orow + ks * 16 + half * 8);
     }
     f32x16 dq[4];
 #pragma unroll
@@ -604,9 +607,9 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
 }
 
 bool flash_shape_ok(int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim, int64_t row, int64_t head,
-                    int64_t batch_stride) {
+                    int64_t batch_stride, int64_t orow, int64_t obatch) {
     return batch > 0 && heads > 0 && tokens >= 4 && tokens % 4 == 0 && head_dim == kHD && row % 8 == 0 &&
-           head % 8 == 0 && batch_stride % 8 == 0 && batch * heads <= (1 << 20) && tokens <= (1 << 20);
+           head % 8 == 0 && batch_stride % 8 == 0 && orow % 8 == 0 && obatch % 8 == 0 && batch * heads <= (1 << 20) && tokens <= (1 << 20);
 }
 
 }  // namespace
@@ -616,13 +619,14 @@ extern "C" {
 int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype, const float* alibi,
                           const int32_t* valid, void* o, float* lse, int64_t batch, int64_t heads, int64_t tokens,
                           int64_t head_dim, int64_t row_stride, int64_t head_stride, int64_t batch_stride,
-                          br_stream_t stream) {
+                          int64_t o_row_stride, int64_t o_batch_stride, br_stream_t stream) {
     if (batch < 0 || heads <= 0 || tokens <= 0 || head_dim <= 0) return BR_ERR_ATTR;
     if (batch == 0) return BR_OK;
     if (!q || !k || !v || !alibi || !valid) return BR_ERR_INPUT;
     if (!o || !lse) return BR_ERR_OUTPUT;
     if ((dtype != BR_F16 && dtype != BR_BF16) ||
-        !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride) || !aligned16(q) ||
+        !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride, o_row_stride,
+                        o_batch_stride) || !aligned16(q) ||
         !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(alibi))
         return BR_ERR_TODO;
     FlashArgs a = {};
@@ -636,6 +640,8 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
     a.row = row_stride;
     a.head = head_stride;
     a.batch_stride = batch_stride;
+    a.orow = o_row_stride;
+    a.obatch = o_batch_stride;
     a.heads = (int)heads;
     a.tokens = (int)tokens;
     a.batch_heads = (int)(batch * heads);
@@ -652,13 +658,15 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
 int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, int dtype,
                           const float* alibi, const int32_t* valid, const float* lse, float* delta, float* dq,
                           float* dk, float* dv, int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim,
-                          int64_t row_stride, int64_t head_stride, int64_t batch_stride, br_stream_t stream) {
+                          int64_t row_stride, int64_t head_stride, int64_t batch_stride, int64_t o_row_stride,
+                          int64_t o_batch_stride, br_stream_t stream) {
     if (batch < 0 || heads <= 0 || tokens <= 0 || head_dim <= 0) return BR_ERR_ATTR;
     if (batch == 0) return BR_OK;
     if (!q || !k || !v || !o || !d_o || !alibi || !valid || !lse) return BR_ERR_INPUT;
     if (!delta || !dq || !dk || !dv) return BR_ERR_OUTPUT;
     if ((dtype != BR_F16 && dtype != BR_BF16) ||
-        !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride) || !aligned16(q) ||
+        !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride, o_row_stride,
+                        o_batch_stride) || !aligned16(q) ||
         !aligned16(k) || !aligned16(v) || !aligned16(o) || !aligned16(d_o) || !aligned16(alibi) || !aligned16(dq) ||
         !aligned16(dk) || !aligned16(dv))
         return BR_ERR_TODO;
@@ -678,6 +686,8 @@ int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     a.row = row_stride;
     a.head = head_stride;
     a.batch_stride = batch_stride;
+    a.orow = o_row_stride;
+    a.obatch = o_batch_stride;
     a.heads = (int)heads;
     a.tokens = (int)tokens;
     a.batch_heads = (int)(batch * heads);

@@ -286,9 +286,12 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
  * key < valid[b], else -FLT_MAX: the table of train_bloom.cpp:73-90 for a batch
  * whose sequences are padded on the right (valid = number of real tokens; a
  * sequence with valid == 0 gets uniform probabilities, as the chain gives).
- * q, k, v, o: fp16 / bf16 (dtype), element (b, t, h, d) at
- * b * batch_stride + t * row_stride + h * head_stride + d, so both
- * [B, T, heads, 128] (the projections' own output) and [B, heads, T, 128] work.
+ * q, k, v, o: fp16 / bf16 (dtype); element (b, t, h, d) of q, k, v at
+ * b * batch_stride + t * row_stride + h * head_stride + d, of o at
+ * b * o_batch_stride + t * o_row_stride + h * head_stride + d.  So
+ * [B, T, heads, 128] (the projections' own output), [B, heads, T, 128] and a
+ * packed [B, T, 3, heads, 128] projection (q, k, v pointing at its thirds,
+ * row_stride = 3 * heads * 128) all work without a transpose.
  * alibi: fp32 [heads, tokens] (br_hip_alibi_table); valid: device int32 [batch].
  * lse[batch, heads, tokens] receives log sum exp of each score row, which the
  * backward needs.  Probabilities are rounded to `dtype` before the product
@@ -297,14 +300,15 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
 int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype, const float* alibi,
                           const int32_t* valid, void* o, float* lse, int64_t batch, int64_t heads,
                           int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
-                          int64_t batch_stride, br_stream_t stream);
+                          int64_t batch_stride, int64_t o_row_stride, int64_t o_batch_stride,
+                          br_stream_t stream);
 
 /* Backward of br_hip_flash_attn_fwd: the chain op_attn_backward
  * (cuda_tensor.cpp:830-888), op_softmax_backward (:890-918) and op_qk_backward
  * (:1004-1063) of train.words:217-226 without the [batch, heads, tokens, tokens]
  * tensors: probabilities are recomputed from q, k and lse.  o is the forward's
- * output, d_o its gradient (both `dtype`, same strides as q, k, v); dq, dk, dv
- * are fp32 with the same element strides.  delta: fp32 scratch of
+ * output, d_o its gradient (both `dtype`, o's strides); dq, dk, dv are fp32
+ * with the element strides of q, k, v.  delta: fp32 scratch of
  * batch * heads * tokens entries (receives rowsum(d_o * o)).  Deterministic: one
  * pass accumulates dk / dv per key block, a second one dq per query block.
  * Same shape limits as the forward (BR_ERR_TODO otherwise). */
@@ -312,7 +316,8 @@ int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
                           int dtype, const float* alibi, const int32_t* valid, const float* lse,
                           float* delta, float* dq, float* dk, float* dv, int64_t batch, int64_t heads,
                           int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
-                          int64_t batch_stride, br_stream_t stream);
+                          int64_t batch_stride, int64_t o_row_stride, int64_t o_batch_stride,
+                          br_stream_t stream);
 
 /* ---- optimizer ---------------------------------------------------------- */
 /* One AdamW step (decoupled weight decay) over n parameters, all arithmetic in

@@ -56,14 +56,22 @@ def test_flash_forward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype)
     o = torch.zeros((b, t, nh, HD), dtype=tdtype, device="cuda")
     lse = empty((b, nh, t))
     call("br_hip_flash_attn_fwd", ptr(dq), ptr(dk), ptr(dv), dtype, ptr(alibi), ptr(dvalid), ptr(o), ptr(lse), b, nh,
-         t, HD, nh * HD, HD, t * nh * HD, stream())
+         t, HD, nh * HD, HD, t * nh * HD, nh * HD, t * nh * HD, stream())
     assert_close(host(o.float()), o_ref, TOL[dtype], "context")
     # the same through [B, NH, T, HD] strides
     zq, zk, zv = (x.permute(0, 2, 1, 3).contiguous() for x in (dq, dk, dv))
     zo = torch.zeros((b, nh, t, HD), dtype=tdtype, device="cuda")
     call("br_hip_flash_attn_fwd", ptr(zq), ptr(zk), ptr(zv), dtype, ptr(alibi), ptr(dvalid), ptr(zo), ptr(lse), b, nh,
-         t, HD, HD, t * HD, nh * t * HD, stream())
+         t, HD, HD, t * HD, nh * t * HD, HD, nh * t * HD, stream())
     assert torch.equal(zo.permute(0, 2, 1, 3), o)
+    # packed [B, T, 3, NH, HD] projection read through strides, o dense
+    packed = torch.stack([dq, dk, dv], dim=2).contiguous()
+    po = torch.zeros((b, t, nh, HD), dtype=tdtype, device="cuda")
+    h3 = 3 * nh * HD
+    call("br_hip_flash_attn_fwd", ptr(packed), ctypes.c_void_p(packed.data_ptr() + 2 * nh * HD),
+         ctypes.c_void_p(packed.data_ptr() + 4 * nh * HD), dtype, ptr(alibi), ptr(dvalid), ptr(po), ptr(lse), b, nh, t,
+         HD, h3, HD, t * h3, nh * HD, t * nh * HD, stream())
+    assert torch.equal(po, o)
     # log-sum-exp rows: exp(s - lse) must be the reference probabilities' normaliser
     s = np.einsum("bqhd,bkhd->bhqk", q.float().numpy().astype(np.float64), k.float().numpy().astype(np.float64))
     s = s / np.sqrt(HD) + orc.alibi(nh, t).astype(np.float64)[None, :, None, :]
@@ -82,12 +90,12 @@ def test_flash_forward_declines_unsupported_shapes():
     f = empty(4096)
     i = torch.ones(4, dtype=torch.int32, device="cuda")
     ok = (ptr(t), ptr(t), ptr(t), F16, ptr(f), ptr(i), ptr(t), ptr(f))
-    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 8, 64, 64, 64, 512, stream()) == -1      # head size 64
-    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 6, 128, 128, 128, 768, stream()) == -1   # tokens % 4
+    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 8, 64, 64, 64, 512, 64, 512, stream()) == -1      # head size 64
+    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 6, 128, 128, 128, 768, 128, 768, stream()) == -1  # tokens % 4
     assert lib.br_hip_flash_attn_fwd(ptr(t), ptr(t), ptr(t), hip.F32, ptr(f), ptr(i), ptr(t), ptr(f), 1, 1, 8, 128,
-                                     128, 128, 1024, stream()) == -1
+                                     128, 128, 1024, 128, 1024, stream()) == -1
     assert lib.br_hip_flash_attn_fwd(None, ptr(t), ptr(t), F16, ptr(f), ptr(i), ptr(t), ptr(f), 1, 1, 8, 128, 128,
-                                     128, 1024, stream()) == -2
+                                     128, 1024, 128, 1024, stream()) == -2
     torch.cuda.synchronize()
 
 
@@ -116,7 +124,7 @@ def test_flash_backward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype
     dvalid = dev(np.asarray(valid, np.int32))
     o = torch.zeros((b, t, nh, HD), dtype=tdtype, device="cuda")
     lse, delta = empty((b, nh, t)), empty((b, nh, t))
-    strides = (b, nh, t, HD, nh * HD, HD, t * nh * HD)
+    strides = (b, nh, t, HD, nh * HD, HD, t * nh * HD, nh * HD, t * nh * HD)
     call("br_hip_flash_attn_fwd", ptr(dq_), ptr(dk_), ptr(dv_), dtype, ptr(alibi), ptr(dvalid), ptr(o), ptr(lse),
          *strides, stream())
     gq, gk, gv = (torch.full((b, t, nh, HD), 7.0, device="cuda") for _ in range(3))
@@ -125,6 +133,15 @@ def test_flash_backward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype
     assert_close(host(gv), dv_ref, TOL[dtype], "dv")
     assert_close(host(gq), dq_ref, TOL[dtype], "dq")
     assert_close(host(gk), dk_ref, TOL[dtype], "dk")
+    # the same from a packed projection, gradients packed likewise
+    packed = torch.stack([dq_, dk_, dv_], dim=2).contiguous()
+    gp = torch.full((b, t, 3, nh, HD), 7.0, device="cuda")
+    h1, h3 = nh * HD, 3 * nh * HD
+    at = lambda x, off: ctypes.c_void_p(x.data_ptr() + off)
+    call("br_hip_flash_attn_bwd", ptr(packed), at(packed, 2 * h1), at(packed, 4 * h1), ptr(o), ptr(dg), dtype,
+         ptr(alibi), ptr(dvalid), ptr(lse), ptr(delta), ptr(gp), at(gp, 4 * h1), at(gp, 8 * h1), b, nh, t, HD, h3, HD,
+         t * h3, h1, t * h1, stream())
+    assert torch.equal(gp[:, :, 0], gq) and torch.equal(gp[:, :, 1], gk) and torch.equal(gp[:, :, 2], gv)
     # keys in the padding receive exactly zero (when the sequence is not empty)
     for bi in range(b):
         if 0 < valid[bi] < t:
