@@ -19,6 +19,10 @@
  *   softmax family         row sums, shift invariance, finite differences
  *   loss head              reference fixtures (ids/mask) brute force, FD
  *   fetch_data pieces      reference fixtures, closed-form ALiBi slopes
+ *   embedding scatter-add  (not in the reference) np.add.at, one-hot product,
+ *                          torch autograd of the tied table
+ *   AdamW (oracle/__init__.py, numpy; not in the reference)
+ *                          torch.optim.AdamW over five steps
  * The arithmetic of cuDNN / cuBLASLt / OpenBLAS that the reference calls is
  * not vendored there and no version is pinned; those calls are restated from
  * their published definitions (softmax, broadcast add, column sum, SGEMM).
