@@ -38,6 +38,8 @@
 
 #include <float.h>
 
+#include <type_traits>
+
 using namespace brk;
 using namespace brk::gemm16;
 
@@ -120,6 +122,38 @@ __device__ __forceinline__ u32x4 frag_cols(const lds_byte* tile, int d0, int ra,
     return mk4(l2.x, l2.y, h2.x, h2.y);
 }
 
+// The same two reads with every lane-dependent part of the address computed
+// once (FragOffsets) and everything else a compile-time constant, so that the
+// reads inside the tile loops need no address arithmetic at all.
+struct FragOffsets {
+    unsigned rows[8];            // frag_rows(tile, 0, ks, lane) - tile
+    unsigned cols_lo[4], cols_hi[4];  // frag_cols(tile, 32 * db, 4 * half, 4 * half + 8, lane) - tile
+    __device__ __forceinline__ explicit FragOffsets(int lane) {
+        const int i = lane & 15, half = lane >> 5;
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) rows[ks] = slot(lane & 31, ks * 2 + half);
+#pragma unroll
+        for (int db = 0; db < 4; db++) {
+            const int d = db * 32 + ((lane >> 4) & 1) * 16 + (i & 3) * 4;
+            const int ja = half * 4 + (i >> 2);
+            cols_lo[db] = slot(ja, d >> 3) + (d & 7) * 2;
+            cols_hi[db] = slot(ja + 8, d >> 3) + (d & 7) * 2;
+        }
+    }
+    // rows r0 .. r0 + 31 (r0 a multiple of 32) of the tile at byte offset `tile`
+    __device__ __forceinline__ u32x4 frag_rows(const lds_byte* lds, int tile, int r0, int ks) const {
+        return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(lds + rows[ks] + (tile + r0 * 256));
+    }
+    // tile rows r16 + 4 * half + 0..3 and + 8 (r16 a multiple of 16), d block db
+    __device__ __forceinline__ u32x4 frag_cols(const lds_byte* lds, int tile, int db, int r16) const {
+        typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lds + cols_lo[db] + (tile + r16 * 256)));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lds + cols_hi[db] + (tile + r16 * 256)));
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        return mk4(l2.x, l2.y, h2.x, h2.y);
+    }
+};
+
 // Row index (within a 32-row accumulator block) of accumulator element v.
 __device__ __forceinline__ int acc_row(int v, int lane) { return (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3); }
 
@@ -174,7 +208,8 @@ struct StageLoader {
 template <int CT>
 __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+    const int lane = threadIdx.x & 63, half = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: branches on it are scalar
     // workgroups are numbered longest first: the query tiles with the most
     // visible keys of every (batch, head), then the next ones, ...
     const int tiles_q = (a.tokens + kBQ - 1) / kBQ;
@@ -204,17 +239,18 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
     // keys this wave's queries can see (a wave may idle through the last tiles)
     const int wave_keys = visible_keys(q0 + 32, valid, a.tokens);
 
+    const FragOffsets fo(lane);
+    const lds_byte* ldsb = (const lds_byte*)lds;
     StageLoader ld;
     ld.fetch(a.k + base, a.v + base, alibi_row, a.row, 0, a.tokens);
     ld.store(lds);
     if (ntiles > 1) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, kBK, a.tokens);
     __syncthreads();
-    for (int t = 0; t < ntiles; t++) {
+    // one key tile; the stage is a compile-time constant so that every LDS
+    // address is a per-lane offset computed once plus an immediate
+    auto tile_step = [&](auto stage_c, int t) {
+        constexpr int kStage = decltype(stage_c)::value * kStageBytes;
         const int k0 = t * kBK;
-        const unsigned char* stage = lds + (t & 1) * kStageBytes;
-        const lds_byte* tk = (const lds_byte*)stage;
-        const lds_byte* tv = (const lds_byte*)(stage + kTileBytes);
-        const float* tb = reinterpret_cast<const float*>(stage + 2 * kTileBytes);
         if (k0 < wave_keys) {
             f32x16 s[2];
 #pragma unroll
@@ -223,31 +259,42 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
                 for (int v = 0; v < 16; v++) s[kb][v] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++)
-                    s[kb] = Cvt<CT>::mfma(frag_rows(tk, kb * 32, ks, lane), qf[ks], s[kb]);
+                    s[kb] = Cvt<CT>::mfma(fo.frag_rows(ldsb, kStage, kb * 32, ks), qf[ks], s[kb]);
             }
-            // tiles wholly below the diagonal and inside the sequence need no mask
-            const bool open = k0 + kBK - 1 <= q0 && k0 + kBK <= valid;
+            const float* tb = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + half * 4;
             float mt = -INFINITY;
+            // tiles wholly below the diagonal and inside the sequence need no mask
+            if (k0 + kBK - 1 <= q0 && k0 + kBK <= valid) {
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int kk = kb * 32 + g * 8 + half * 4;
-                    const float4 bv = *reinterpret_cast<const float4*>(tb + kk);
-                    const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+                    for (int g = 0; g < 4; g++) {
+                        const float4 bv = *reinterpret_cast<const float4*>(tb + kb * 32 + g * 8);
+                        const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        float x;
-                        if (open) {
-                            x = s[kb][g * 4 + j] * a.scale;
+                        for (int j = 0; j < 4; j++) {
+                            float x = s[kb][g * 4 + j] * a.scale;
                             x += bb[j];
-                        } else {
-                            x = score(s[kb][g * 4 + j], a.scale, bb[j], query, k0 + kk + j, valid, a.tokens);
+                            s[kb][g * 4 + j] = x;
+                            mt = fmaxf(mt, x);
                         }
-                        s[kb][g * 4 + j] = x;
-                        mt = fmaxf(mt, x);
                     }
-                }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float4 bv = *reinterpret_cast<const float4*>(tb + kb * 32 + g * 8);
+                        const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+                        const int key = k0 + kb * 32 + g * 8 + half * 4;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float x = score(s[kb][g * 4 + j], a.scale, bb[j], query, key + j, valid, a.tokens);
+                            s[kb][g * 4 + j] = x;
+                            mt = fmaxf(mt, x);
+                        }
+                    }
+            }
             mt = fmaxf(mt, xor32(mt));
             const float m_new = fmaxf(m, mt);
             const float alpha = __expf(m - m_new);
@@ -274,19 +321,22 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) p8[e] = s[kb][vb + e];
                 const u32x4 pf = pack8<CT>(p8);
-                const int ra = kb * 32 + (j & 1) * 16 + half * 4;
 #pragma unroll
                 for (int db = 0; db < 4; db++)
-                    o[db] = Cvt<CT>::mfma(frag_cols(tv, db * 32, ra, ra + 8, lane), pf, o[db]);
+                    o[db] = Cvt<CT>::mfma(fo.frag_cols(ldsb, kStage + kTileBytes, db, kb * 32 + (j & 1) * 16), pf, o[db]);
             }
         }
-        // tile t+1 (in registers since the previous iteration) goes into the
-        // other stage, whose last readers passed the barrier of iteration t-1
+        // tile t+1 (in registers since the previous step) goes into the other
+        // stage, whose last readers passed the barrier of step t-1
         if (t + 1 < ntiles) {
-            ld.store(lds + ((t + 1) & 1) * kStageBytes);
+            ld.store(lds + (kStageBytes - kStage));
             if (t + 2 < ntiles) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, k0 + 2 * kBK, a.tokens);
         }
         __syncthreads();
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        tile_step(std::integral_constant<int, 0>(), t);
+        if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
     }
 
     if (query < a.tokens) {
@@ -372,7 +422,8 @@ struct QStageLoader {
 template <int CT>
 __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kQStageBytes];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+    const int lane = threadIdx.x & 63, half = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: branches on it are scalar
     const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
     const int kt = (int)(blockIdx.x / a.batch_heads);  // key tile 0 meets the most queries: longest first
     const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
@@ -404,6 +455,8 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
     const int ntiles = dead_group ? 0 : (a.tokens - q_begin + kBK - 1) / kBK;
     const bool dead_wave = valid > 0 && key0 >= valid;
 
+    const FragOffsets fo(lane);
+    const lds_byte* ldsb = (const lds_byte*)lds;
     QStageLoader ld;
     if (ntiles > 0) {
         ld.fetch(a, base, obase, bh, q_begin);
@@ -411,12 +464,10 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
         if (ntiles > 1) ld.fetch(a, base, obase, bh, q_begin + kBK);
     }
     __syncthreads();
-    for (int t = 0; t < ntiles; t++) {
+    auto tile_step = [&](auto stage_c, int t) {
+        constexpr int kStage = decltype(stage_c)::value * kQStageBytes;
         const int q0 = q_begin + t * kBK;
-        const unsigned char* stage = lds + (t & 1) * kQStageBytes;
-        const lds_byte* tq = (const lds_byte*)stage;
-        const lds_byte* tg = (const lds_byte*)(stage + kTileBytes);
-        const float* tl = reinterpret_cast<const float*>(stage + 2 * kTileBytes);
+        const float* tl = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + half * 4;
         const float* td = tl + kBK;
         // a tile whose queries all precede this wave's keys sees none of them
         if (!dead_wave && !(valid > 0 && q0 + kBK - 1 < key0)) {
@@ -428,30 +479,39 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
                 for (int v = 0; v < 16; v++) s[v] = dp[v] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++) {
-                    s = Cvt<CT>::mfma(frag_rows(tq, qb * 32, ks, lane), kf[ks], s);
-                    dp = Cvt<CT>::mfma(frag_rows(tg, qb * 32, ks, lane), vf[ks], dp);
+                    s = Cvt<CT>::mfma(fo.frag_rows(ldsb, kStage, qb * 32, ks), kf[ks], s);
+                    dp = Cvt<CT>::mfma(fo.frag_rows(ldsb, kStage + kTileBytes, qb * 32, ks), vf[ks], dp);
                 }
+                if (open) {
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int qq = qb * 32 + g * 8 + half * 4;
-                    const float4 l4 = *reinterpret_cast<const float4*>(tl + qq);
-                    const float4 d4 = *reinterpret_cast<const float4*>(td + qq);
-                    const float ll[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
+                    for (int g = 0; g < 4; g++) {
+                        const float4 l4 = *reinterpret_cast<const float4*>(tl + qb * 32 + g * 8);
+                        const float4 d4 = *reinterpret_cast<const float4*>(td + qb * 32 + g * 8);
+                        const float ll[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const int query = q0 + qq + j;
-                        float p;
-                        if (open) {
+                        for (int j = 0; j < 4; j++) {
                             float x = s[g * 4 + j] * a.scale;
                             x += bias;
-                            p = __expf(x - ll[j]);
-                        } else {
-                            const float x = score(s[g * 4 + j], a.scale, bias, query, key, valid, a.tokens);
-                            p = valid > 0 ? __expf(x - ll[j]) : uniform;
-                            p = (query < a.tokens && key < a.tokens) ? p : 0.f;
+                            const float p = __expf(x - ll[j]);
+                            s[g * 4 + j] = p;
+                            dp[g * 4 + j] = p * (dp[g * 4 + j] - dd[j]);
                         }
-                        s[g * 4 + j] = p;
-                        dp[g * 4 + j] = p * (dp[g * 4 + j] - dd[j]);
+                    }
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float4 l4 = *reinterpret_cast<const float4*>(tl + qb * 32 + g * 8);
+                        const float4 d4 = *reinterpret_cast<const float4*>(td + qb * 32 + g * 8);
+                        const float ll[4] = {l4.x, l4.y, l4.z, l4.w}, dd[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const int query = q0 + qb * 32 + g * 8 + half * 4 + j;
+                            const float x = score(s[g * 4 + j], a.scale, bias, query, key, valid, a.tokens);
+                            float p = valid > 0 ? __expf(x - ll[j]) : uniform;
+                            p = (query < a.tokens && key < a.tokens) ? p : 0.f;
+                            s[g * 4 + j] = p;
+                            dp[g * 4 + j] = p * (dp[g * 4 + j] - dd[j]);
+                        }
                     }
                 }
 #pragma unroll
@@ -463,20 +523,23 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
                         s8[e] = dp[j * 8 + e];
                     }
                     const u32x4 pf = pack8<CT>(p8), sf = pack8<CT>(s8);
-                    const int ra = qb * 32 + j * 16 + half * 4;
 #pragma unroll
                     for (int db = 0; db < 4; db++) {
-                        dv[db] = Cvt<CT>::mfma(pf, frag_cols(tg, db * 32, ra, ra + 8, lane), dv[db]);
-                        dk[db] = Cvt<CT>::mfma(sf, frag_cols(tq, db * 32, ra, ra + 8, lane), dk[db]);
+                        dv[db] = Cvt<CT>::mfma(pf, fo.frag_cols(ldsb, kStage + kTileBytes, db, qb * 32 + j * 16), dv[db]);
+                        dk[db] = Cvt<CT>::mfma(sf, fo.frag_cols(ldsb, kStage, db, qb * 32 + j * 16), dk[db]);
                     }
                 }
             }
         }
         if (t + 1 < ntiles) {
-            ld.store(lds + ((t + 1) & 1) * kQStageBytes);
+            ld.store(lds + (kQStageBytes - kStage));
             if (t + 2 < ntiles) ld.fetch(a, base, obase, bh, q0 + 2 * kBK);
         }
         __syncthreads();
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        tile_step(std::integral_constant<int, 0>(), t);
+        if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
     }
 
     // accumulator element v of block db: key key0 + acc_row(v), d = 32 * db + lane % 32
@@ -500,7 +563,8 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
 template <int CT>
 __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, half = lane >> 5;
+    const int lane = threadIdx.x & 63, half = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: branches on it are scalar
     const int tiles_q = (a.tokens + kBQ - 1) / kBQ;
     const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
     const int qt = tiles_q - 1 - (int)(blockIdx.x / a.batch_heads);
@@ -531,17 +595,17 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
     const int ntiles = (nkeys + kBK - 1) / kBK;
     const int wave_keys = visible_keys(q0 + 32, valid, a.tokens);
 
+    const FragOffsets fo(lane);
+    const lds_byte* ldsb = (const lds_byte*)lds;
     StageLoader ld;
     ld.fetch(a.k + base, a.v + base, alibi_row, a.row, 0, a.tokens);
     ld.store(lds);
     if (ntiles > 1) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, kBK, a.tokens);
     __syncthreads();
-    for (int t = 0; t < ntiles; t++) {
+    auto tile_step = [&](auto stage_c, int t) {
+        constexpr int kStage = decltype(stage_c)::value * kStageBytes;
         const int k0 = t * kBK;
-        const unsigned char* stage = lds + (t & 1) * kStageBytes;
-        const lds_byte* tk = (const lds_byte*)stage;
-        const lds_byte* tv = (const lds_byte*)(stage + kTileBytes);
-        const float* tb = reinterpret_cast<const float*>(stage + 2 * kTileBytes);
+        const float* tb = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + half * 4;
         if (k0 < wave_keys) {
             const bool open = k0 + kBK - 1 <= q0 && k0 + kBK <= valid;
 #pragma unroll
@@ -551,27 +615,34 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
                 for (int v = 0; v < 16; v++) s[v] = dp[v] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++) {
-                    s = Cvt<CT>::mfma(frag_rows(tk, kb * 32, ks, lane), qf[ks], s);
-                    dp = Cvt<CT>::mfma(frag_rows(tv, kb * 32, ks, lane), gf[ks], dp);
+                    s = Cvt<CT>::mfma(fo.frag_rows(ldsb, kStage, kb * 32, ks), qf[ks], s);
+                    dp = Cvt<CT>::mfma(fo.frag_rows(ldsb, kStage + kTileBytes, kb * 32, ks), gf[ks], dp);
                 }
+                if (open) {
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int kk = kb * 32 + g * 8 + half * 4;
-                    const float4 bv = *reinterpret_cast<const float4*>(tb + kk);
-                    const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+                    for (int g = 0; g < 4; g++) {
+                        const float4 bv = *reinterpret_cast<const float4*>(tb + kb * 32 + g * 8);
+                        const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        float p;
-                        if (open) {
+                        for (int j = 0; j < 4; j++) {
                             float x = s[g * 4 + j] * a.scale;
                             x += bb[j];
-                            p = __expf(x - lse);
-                        } else {
-                            const float x = score(s[g * 4 + j], a.scale, bb[j], query, k0 + kk + j, valid, a.tokens);
-                            p = valid > 0 ? __expf(x - lse) : uniform;
-                            p = k0 + kk + j < a.tokens ? p : 0.f;
+                            dp[g * 4 + j] = __expf(x - lse) * (dp[g * 4 + j] - delta);
                         }
-                        dp[g * 4 + j] = p * (dp[g * 4 + j] - delta);
+                    }
+                } else {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float4 bv = *reinterpret_cast<const float4*>(tb + kb * 32 + g * 8);
+                        const float bb[4] = {bv.x, bv.y, bv.z, bv.w};
+                        const int key = k0 + kb * 32 + g * 8 + half * 4;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float x = score(s[g * 4 + j], a.scale, bb[j], query, key + j, valid, a.tokens);
+                            float p = valid > 0 ? __expf(x - lse) : uniform;
+                            p = key + j < a.tokens ? p : 0.f;
+                            dp[g * 4 + j] = p * (dp[g * 4 + j] - delta);
+                        }
                     }
                 }
 #pragma unroll
@@ -580,18 +651,21 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
 #pragma unroll
                     for (int e = 0; e < 8; e++) s8[e] = dp[j * 8 + e];
                     const u32x4 sf = pack8<CT>(s8);
-                    const int ra = kb * 32 + j * 16 + half * 4;
 #pragma unroll
                     for (int db = 0; db < 4; db++)
-                        dq[db] = Cvt<CT>::mfma(frag_cols(tk, db * 32, ra, ra + 8, lane), sf, dq[db]);
+                        dq[db] = Cvt<CT>::mfma(fo.frag_cols(ldsb, kStage, db, kb * 32 + j * 16), sf, dq[db]);
                 }
             }
         }
         if (t + 1 < ntiles) {
-            ld.store(lds + ((t + 1) & 1) * kStageBytes);
+            ld.store(lds + (kStageBytes - kStage));
             if (t + 2 < ntiles) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, k0 + 2 * kBK, a.tokens);
         }
         __syncthreads();
+    };
+    for (int t = 0; t < ntiles; t += 2) {
+        tile_step(std::integral_constant<int, 0>(), t);
+        if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
     }
 
     if (query < a.tokens) {
