@@ -680,6 +680,50 @@ ComputingReturn HIPTensor<DT>::op_qk_backward(tensor_t self, tensor_t q, tensor_
     return OP_OK;
 }
 
+ComputingReturn hip_linear_accumulate(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& y) {
+    if (!dev(x) || !dev(w) || !dev(bias) || x->shape().dim() != 3) return OP_INPUT_ERROR;
+    if (!dev_f32(y)) return OP_OUTPUT_ERROR;
+    const int64_t n = (int64_t)(x->shape()[0] * x->shape()[1]);
+    const int64_t in = (int64_t)x->shape()[2];
+    const int64_t out = (int64_t)w->shape()[0];
+    if ((int64_t)w->shape()[1] != in || (int64_t)bias->items() != out) return OP_INPUT_ERROR;
+    if ((int64_t)y->items() != n * out) return OP_OUTPUT_ERROR;
+    BR_OP(product(0, 1, n, out, in, 1.0f, x->data(), code(x), in, 0, w->data(), code(w), in, 0, 1, y->data(), BR_F32,
+                  out, 0, bias_f32(bias, 0), 1, pick_compute({x, w, y})));
+    return OP_OK;
+}
+
+ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& scale, const tensor_t& bias,
+                                           const tensor_t& var, const tensor_t& y, const tensor_t& dscale,
+                                           const tensor_t& dbias, const tensor_t& residual, const tensor_t& din,
+                                           float eps) {
+    bool fast = dev_f32(dy) && dev_f32(scale) && dev_f32(bias) && dev_f32(var) && dev_f32(y) && dev_f32(dscale) &&
+                dev_f32(dbias) && dev_f32(residual) && dev_f32(din) && dy->shape().dim() == 3;
+    if (fast) {
+        const int64_t rows = (int64_t)(dy->shape()[0] * dy->shape()[1]);
+        const int64_t cols = (int64_t)dy->shape()[2];
+        fast = y->items() == dy->items() && (int64_t)var->items() >= rows && din->items() == dy->items() &&
+               residual->items() == dy->items() && (int64_t)dscale->items() == cols && (int64_t)dbias->items() == cols &&
+               (int64_t)scale->items() == cols && (int64_t)bias->items() == cols && din->data() != y->data();
+        if (fast) {
+            const size_t need = br_hip_layernorm_bwd_workspace(rows, cols);
+            void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
+            const int rc = br_hip_layernorm_bwd_residual(
+                static_cast<const float*>(dy->data()), static_cast<const float*>(y->data()),
+                static_cast<const float*>(scale->data()), static_cast<const float*>(bias->data()),
+                static_cast<const float*>(var->data()), static_cast<const float*>(residual->data()),
+                static_cast<float*>(dscale->data()), static_cast<float*>(dbias->data()),
+                static_cast<float*>(din->data()), rows, cols, eps, ws, need, stream());
+            if (rc != BR_ERR_TODO) return done(rc, "br_hip_layernorm_bwd_residual");
+        }
+    }
+    // the two operators; din must then be a buffer of its own
+    if (din->data() == residual->data()) return OP_OUTPUT_ERROR;
+    ComputingReturn r = dy->op_layernorm_backward(dy, scale, bias, var, y, dscale, dbias, din, eps);
+    if (r != OP_OK) return r;
+    return din->op_add(din, residual, din);
+}
+
 template struct HIPTensor<DataType::Float>;
 template struct HIPTensor<DataType::F16>;
 template struct HIPTensor<DataType::BF16>;

@@ -71,4 +71,15 @@ private:
     const bool owner_;
 };
 
+// y += x . w^T + bias: op_linear (cuda_tensor.cpp:146-193) followed by
+// op_add(y, ., y) with the addition done in the product's epilogue; the sum is
+// formed from the same fp32 values, so the bits equal the two operators'.
+ComputingReturn hip_linear_accumulate(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& y);
+// din = layernorm_backward(...) + residual in one pass where the row kernel
+// applies, else the two operators one after the other (din may be residual).
+ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& scale, const tensor_t& bias,
+                                           const tensor_t& var, const tensor_t& y, const tensor_t& dscale,
+                                           const tensor_t& dbias, const tensor_t& residual, const tensor_t& din,
+                                           float eps);
+
 }  // namespace br

@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "br_hip.h"
+#include "hip_tensor.hpp"
 #include "runtime.hpp"
 #include "tensor.hpp"
 
@@ -35,6 +36,12 @@ struct Tensors {
         void run(Stack& stack) override { __VA_ARGS__ }   \
         NWORD_CREATOR_DEFINE_LR(CLS)                      \
     };
+
+// Free-function operators follow the TensorType wrappers' convention: anything
+// but OP_OK is fatal.
+void op_check_word(ComputingReturn r, const char* what) {
+    if (r != OP_OK) br_panic(what);
+}
 
 // True when `dst <- src` is the 16-bit device image of the fp32 device tensor
 // `produced` (src is that very tensor).
@@ -328,6 +335,21 @@ BR_WORD(FlashAttnQkvBackward,
                                        f.tokens * 3 * hidden, hidden, f.tokens * hidden, ComputingContext::stream));
 )
 
+// Two operator pairs of the model scripts with the addition folded into the
+// producing kernel (same bits as the pair; no counterpart word in the reference):
+// ( x w b y -- )   y += x . w^T + b          `op.linear` into a temporary + `op.add`
+BR_WORD(LinearAdd,
+    Tensors<4> a(stack);
+    op_check_word(hip_linear_accumulate(a[0], a[1], a[2], a[3]), "op.linear_add");
+)
+// ( dy scale bias var y dscale dbias residual din eps -- )   din = dLN + residual
+BR_WORD(LayernormBackwardAdd,
+    const float eps = (float)stack.pop_number();
+    Tensors<9> a(stack);
+    op_check_word(hip_layernorm_backward_add(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], a[8], eps),
+                  "op.layernorm_backward_add");
+)
+
 // AdamW on one parameter tensor.  The reference stops at the gradients; these
 // two words are what a training loop runs after them.
 // ( param [master] grad m v lr beta1 beta2 eps weight_decay step -- )
@@ -412,6 +434,8 @@ void load_nn_words(Enviroment& env) {
         {"op.softmax_backward", SoftmaxBackward::creator},
         {"op.softmax_attn_backward", SoftmaxAttnBackward::creator},
         {"op.qk_backward", QueryKeyBackward::creator},
+        {"op.linear_add", LinearAdd::creator},
+        {"op.layernorm_backward_add", LayernormBackwardAdd::creator},
         {"op.flash_attn", FlashAttn::creator},
         {"op.flash_attn_backward", FlashAttnBackward::creator},
         {"op.flash_attn_qkv", FlashAttnQkv::creator},

@@ -111,13 +111,13 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic(const float* x, const f
 
 // --------------------------------------------------------------- backward
 template <int VPT>
-__global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* __restrict__ dy, const float* __restrict__ y,
+__global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* dy, const float* __restrict__ y,
                                                        const float* __restrict__ gamma,
                                                        const float* __restrict__ beta,
-                                                       const float* __restrict__ var, float* __restrict__ dx,
+                                                       const float* __restrict__ var, float* dx,
                                                        float* __restrict__ part_dgamma,
                                                        float* __restrict__ part_dbeta, int64_t rows, int cols4,
-                                                       float eps, float inv_cols) {
+                                                       float eps, float inv_cols, const float* residual) {
     __shared__ float lds[2][2 * kWaves];
     float4 g[VPT], ginv[VPT], b[VPT], acc_g[VPT], acc_b[VPT];
 #pragma unroll
@@ -152,6 +152,17 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* __restrict__ 
         if (next < rows) request(nd, nxh, next);
         // stored var already holds eps; the backward adds eps once more
         const float rstd = 1.0f / sqrtf(var[row] + eps);
+        // optional residual gradient added to dx (dx may be the same buffer):
+        // requested here so that its latency hides behind the row reduction
+        float4 res[VPT];
+        if (residual) {
+            const float4* rr = reinterpret_cast<const float4*>(residual) + row * cols4;
+#pragma unroll
+            for (int i = 0; i < VPT; i++) {
+                const int idx = threadIdx.x + i * kBlock;
+                res[i] = idx < cols4 ? rr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
         float s[2] = {0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
@@ -179,6 +190,11 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* __restrict__ 
                 o.y = (d[i].y - m1 - xh[i].y * m2) * rstd;
                 o.z = (d[i].z - m1 - xh[i].z * m2) * rstd;
                 o.w = (d[i].w - m1 - xh[i].w * m2) * rstd;
+                if (residual) {
+                    // dx is rounded to fp32 before the add, as a separate add kernel would see it
+                    asm volatile("" : "+v"(o.x), "+v"(o.y), "+v"(o.z), "+v"(o.w));
+                    o.x += res[i].x; o.y += res[i].y; o.z += res[i].z; o.w += res[i].w;
+                }
                 dxr[idx] = o;
             }
         }
@@ -388,9 +404,10 @@ size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols) {
     return (size_t)(2 * parts * cols) * sizeof(float);
 }
 
-int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, const float* beta,
-                         const float* var, float* dgamma, float* dbeta, float* dx, int64_t rows, int64_t cols,
-                         float eps, void* workspace, size_t workspace_bytes, br_stream_t stream) {
+static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamma, const float* beta,
+                              const float* var, const float* residual, float* dgamma, float* dbeta, float* dx,
+                              int64_t rows, int64_t cols, float eps, void* workspace, size_t workspace_bytes,
+                              br_stream_t stream) {
     if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
     if (!dgamma || !dbeta) return BR_ERR_OUTPUT;
     if (rows == 0) {
@@ -403,20 +420,27 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, co
     hipStream_t st = as_stream(stream);
     int parts;
     float* part_g = (float*)workspace;
-    if (regs_path_ok(cols, dy, y, gamma, beta, dx) && aligned16(workspace)) {
+    const bool regs = regs_path_ok(cols, dy, y, gamma, beta, dx) && aligned16(workspace) &&
+                      (!residual || aligned16(residual));
+    if (residual && !regs) return BR_ERR_TODO;  // only the register path adds the residual
+    if (regs) {
         parts = bwd_parts(rows);
         float* part_b = part_g + (int64_t)parts * cols;
         const int cols4 = (int)(cols / 4);
         const float inv = 1.0f / (float)cols;
         const int vpt = (cols4 + kBlock - 1) / kBlock;
         if (vpt <= 1)
-            ln_bwd_regs<1><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+            ln_bwd_regs<1><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
+                                                     residual);
         else if (vpt <= 2)
-            ln_bwd_regs<2><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+            ln_bwd_regs<2><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
+                                                     residual);
         else if (vpt <= 4)
-            ln_bwd_regs<4><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+            ln_bwd_regs<4><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
+                                                     residual);
         else
-            ln_bwd_regs<8><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv);
+            ln_bwd_regs<8><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
+                                                     residual);
         BR_HIP_LAUNCH_CHECK();
         if (aligned16(dgamma) && aligned16(dbeta))
             ln_bwd_finalize_x4<<<(unsigned)((cols4 + 15) / 16), 1024, 0, st>>>(
@@ -438,6 +462,23 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, co
     }
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
+}
+
+int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, const float* beta,
+                         const float* var, float* dgamma, float* dbeta, float* dx, int64_t rows, int64_t cols,
+                         float eps, void* workspace, size_t workspace_bytes, br_stream_t stream) {
+    return layernorm_bwd_impl(dy, y, gamma, beta, var, nullptr, dgamma, dbeta, dx, rows, cols, eps, workspace,
+                              workspace_bytes, stream);
+}
+
+int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* gamma, const float* beta,
+                                  const float* var, const float* residual, float* dgamma, float* dbeta, float* dx,
+                                  int64_t rows, int64_t cols, float eps, void* workspace, size_t workspace_bytes,
+                                  br_stream_t stream) {
+    if (rows > 0 && !residual) return BR_ERR_INPUT;
+    if (rows == 0) residual = nullptr;
+    return layernorm_bwd_impl(dy, y, gamma, beta, var, residual, dgamma, dbeta, dx, rows, cols, eps, workspace,
+                              workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -163,6 +163,18 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma,
                          float* dx, int64_t rows, int64_t cols, float eps, void* workspace,
                          size_t workspace_bytes, br_stream_t stream);
 
+/* The same backward with a residual gradient added to the input gradient:
+ * dx = layernorm_backward(...) + residual, the `op.layernorm_backward` +
+ * `op.add` pair of train.words:207-208 and :240-243 (cuda_tensor.cpp:699-727
+ * followed by :206-232) in one pass.  dx is rounded to fp32 before the add, so
+ * the result equals the two operators' bit for bit; dx may be the residual's
+ * or dy's own buffer (a row is read completely before it is written).  BR_ERR_TODO when the shape needs the general kernels. */
+int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* gamma,
+                                  const float* beta, const float* var, const float* residual,
+                                  float* dgamma, float* dbeta, float* dx, int64_t rows,
+                                  int64_t cols, float eps, void* workspace, size_t workspace_bytes,
+                                  br_stream_t stream);
+
 /* ---- softmax family ---------------------------------------------------- */
 /* cudnnSoftmaxForward(ACCURATE, INSTANCE) at cuda_tensor.cpp:332-356 and
  * cudnnSoftmaxBackward at :890-918.  y may alias x; dx may alias dy. */

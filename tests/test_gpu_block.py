@@ -313,3 +313,48 @@ def test_block_with_fused_attention_matches_oracle(runtime, mode, tol):
     env.execute("layer_forward_mixed op.sync")
     assert_close(flash_out, env.read("xa"), tol, "flash vs operator chain")
     env.close()
+
+
+def test_linear_add_and_layernorm_backward_add_words_equal_the_operator_pairs(runtime):
+    """`op.linear_add` = `op.linear` into a temporary + `op.add`;
+    `op.layernorm_backward_add` = `op.layernorm_backward` + `op.add`: same bits,
+    in fp32 and fp16 product modes, also on a width the row kernel declines."""
+    rng = np.random.default_rng(8)
+    for mode, hidden in (("f32", 256), ("f16", 256), ("f32", 102)):
+        b, t = 2, 24
+        env = host.Env(1)
+        try:
+            env.execute("'%s' op.gemm_precision" % mode)
+            wdt = "f16" if mode == "f16" else "float"
+            env.execute("%d %d %d 3 'cuda' '%s' op.create 'x' !" % (b, t, 4 * hidden, wdt))
+            env.execute("%d %d 2 'cuda' '%s' op.create 'w' !  %d 1 'cuda' 'float' op.create 'bias' !"
+                        % (hidden, 4 * hidden, wdt, hidden))
+            for n in ("y", "tmp", "acc", "dy", "ln", "res", "din", "din2"):
+                env.execute("%d %d %d 3 'cuda' 'float' op.create '%s' !" % (b, t, hidden, n))
+            for n in ("var", "g", "be", "dg", "db", "dg2", "db2"):
+                env.execute("%d 1 'cuda' 'float' op.create '%s' !" % (max(hidden, b * t), n))
+            env.execute("%d 1 'cuda' 'float' op.create 'gam' !  %d 1 'cuda' 'float' op.create 'bet' !" % (hidden, hidden))
+            env.execute("%d 1 'cuda' 'float' op.create 'dgam' !  %d 1 'cuda' 'float' op.create 'dbet' !" % (hidden, hidden))
+            env.execute("%d 1 'cuda' 'float' op.create 'dgam2' !  %d 1 'cuda' 'float' op.create 'dbet2' !" % (hidden, hidden))
+            env.write("x", rng.standard_normal((b, t, 4 * hidden)).astype(np.float32))
+            env.write("w", (0.05 * rng.standard_normal((hidden, 4 * hidden))).astype(np.float32))
+            env.write("bias", rng.standard_normal(hidden).astype(np.float32))
+            acc0 = rng.standard_normal((b, t, hidden)).astype(np.float32)
+            env.write("acc", acc0)
+            env.execute("'x' @ 'w' @ 'bias' @ 'tmp' @ op.linear  'acc' @ 'tmp' @ 'y' @ op.add")
+            env.execute("'x' @ 'w' @ 'bias' @ 'acc' @ op.linear_add")
+            assert np.array_equal(env.read("acc"), env.read("y")), mode
+
+            env.write("gam", (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32))
+            env.write("bet", (0.1 * rng.standard_normal(hidden)).astype(np.float32))
+            env.write("dy", rng.standard_normal((b, t, hidden)).astype(np.float32))
+            env.write("res", rng.standard_normal((b, t, hidden)).astype(np.float32))
+            env.execute("'acc' @ 'g' @ 'var' @ 'gam' @ 'bet' @ 'ln' @ 1e-5 op.layernorm")
+            env.execute("'dy' @ 'gam' @ 'bet' @ 'var' @ 'ln' @ 'dgam' @ 'dbet' @ 'din' @ 1e-5 op.layernorm_backward"
+                        "  'din' @ 'res' @ 'din' @ op.add")
+            env.execute("'dy' @ 'gam' @ 'bet' @ 'var' @ 'ln' @ 'dgam2' @ 'dbet2' @ 'res' @ 'din2' @ 1e-5 "
+                        "op.layernorm_backward_add")
+            assert np.array_equal(env.read("din2"), env.read("din")), (mode, hidden)
+            assert np.array_equal(env.read("dgam2"), env.read("dgam")) and np.array_equal(env.read("dbet2"), env.read("dbet"))
+        finally:
+            env.close()

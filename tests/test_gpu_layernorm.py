@@ -136,3 +136,32 @@ def test_layernorm_fwd_with_16_bit_copy_declines_what_the_row_kernel_cannot_do()
     assert lib.br_hip_layernorm_fwd_copy16(ptr(t), ptr(g), ptr(g), ptr(t), None, F16, None, None, rows, 1000, 1e-5,
                                            stream()) == -3
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (37, 1024), (5, 8192)])
+def test_layernorm_bwd_with_residual_equals_backward_then_add(rows, cols):
+    """dx = layernorm_backward(...) + residual in one pass: bit for bit the
+    plain backward followed by an fp32 add, also when dx is written over the
+    residual or over dy; dgamma / dbeta are unchanged."""
+    print("case rows=%d cols=%d" % (rows, cols), flush=True)
+    x, g, b, dy = make(rows, cols, seed=5)
+    res = np.random.default_rng(6).standard_normal((rows, cols)).astype(np.float32)
+    eps = 1e-5
+    y_ref, _, var_ref = orc.layernorm_fwd(x, g, b, eps)
+    dx_plain, dg_plain, db_plain = run_bwd(dy, y_ref, g, b, var_ref, eps)
+    want = dx_plain + res
+    ws = workspace(hip.load().br_hip_layernorm_bwd_workspace(rows, cols))
+    for alias in ("none", "residual", "dy"):
+        t_dy, t_y, t_g, t_b, t_var, t_res = (dev(a) for a in (dy, y_ref, g, b, var_ref, res))
+        dgam, dbet = empty(cols), empty(cols)
+        out = {"none": empty((rows, cols)), "residual": t_res, "dy": t_dy}[alias]
+        call("br_hip_layernorm_bwd_residual", ptr(t_dy), ptr(t_y), ptr(t_g), ptr(t_b), ptr(t_var), ptr(t_res),
+             ptr(dgam), ptr(dbet), ptr(out), rows, cols, eps, ptr(ws), ws.numel(), stream())
+        assert np.array_equal(host(out), want), alias
+        assert np.array_equal(host(dgam), dg_plain) and np.array_equal(host(dbet), db_plain), alias
+    # shapes the row kernel cannot take are declined
+    t = empty(4 * 1001)
+    gg = empty(1001)
+    assert hip.load().br_hip_layernorm_bwd_residual(ptr(t), ptr(t), ptr(gg), ptr(gg), ptr(gg), ptr(t), ptr(gg), ptr(gg),
+                                                    ptr(t), 4, 1001, eps, ptr(ws), ws.numel(), stream()) == -1
+    torch.cuda.synchronize()
