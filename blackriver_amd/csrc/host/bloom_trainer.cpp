@@ -31,7 +31,7 @@ bool BloomTrainer::mixed() const {
 }
 
 bool BloomTrainer::flash() const {
-    return cfg_.fused_attention && mixed() && cfg_.hidden / cfg_.heads == 128 && cfg_.tokens % 4 == 0;
+    return cfg_.fused_attention && mixed() && cfg_.hidden / cfg_.heads == 128;
 }
 
 int64_t BloomTrainer::model_arena_floats() const {

@@ -55,7 +55,7 @@ public:
     int64_t block_arena_floats() const;
     int64_t model_arena_floats() const;
     bool mixed() const;
-    // fused attention is on and applies: 16-bit operand buffers, head size 128, tokens % 4 == 0
+    // fused attention is on and applies: 16-bit operand buffers, head size 128
     bool flash() const;
     std::string setup_script() const;
     std::string step_script() const;

@@ -682,7 +682,7 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
 
 bool flash_shape_ok(int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim, int64_t row, int64_t head,
                     int64_t batch_stride, int64_t orow, int64_t obatch) {
-    return batch > 0 && heads > 0 && tokens >= 4 && tokens % 4 == 0 && head_dim == kHD && row % 8 == 0 &&
+    return batch > 0 && heads > 0 && tokens >= 1 && head_dim == kHD && row % 8 == 0 &&
            head % 8 == 0 && batch_stride % 8 == 0 && orow % 8 == 0 && obatch % 8 == 0 && batch * heads <= (1 << 20) && tokens <= (1 << 20);
 }
 

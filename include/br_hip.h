@@ -307,7 +307,7 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
  * alibi: fp32 [heads, tokens] (br_hip_alibi_table); valid: device int32 [batch].
  * lse[batch, heads, tokens] receives log sum exp of each score row, which the
  * backward needs.  Probabilities are rounded to `dtype` before the product
- * with v.  BR_ERR_TODO unless head_dim == 128, tokens % 4 == 0, strides % 8 == 0
+ * with v.  BR_ERR_TODO unless head_dim == 128, strides % 8 == 0
  * and 16-byte aligned bases: callers then run the unfused chain. */
 int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype, const float* alibi,
                           const int32_t* valid, void* o, float* lse, int64_t batch, int64_t heads,

@@ -101,7 +101,7 @@ int br_bloom_model_create(br_env_t* env, int layers, int64_t batch, int64_t toke
                           const char* gemm_precision);
 /* Before br_bloom_model_create: whether attention runs as one fused kernel per
  * direction (default; applies with 16-bit weights multiplied in their own
- * type, head size 128 and tokens % 4 == 0) or as the reference's operator
+ * type and head size 128) or as the reference's operator
  * chain through [batch, heads, tokens, tokens] tensors. */
 int br_bloom_model_set_fused_attention(br_env_t* env, int on);
 int br_bloom_model_init(br_env_t* env, uint64_t seed, float std);

@@ -44,6 +44,7 @@ def reference_forward(q, k, v, valid):
     (2, 3, 200, (200, 1)),        # tokens not a multiple of the tile sizes; a one-token sequence
     (2, 2, 132, (0, 77)),         # an empty sequence: uniform probabilities, as the unfused chain gives
     (1, 1, 4, (3,)),
+    (1, 2, 37, (30,)),            # odd token count
 ])
 def test_flash_forward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype):
     print("case b=%d nh=%d t=%d valid=%s dtype=%d" % (b, nh, t, valid, dtype), flush=True)
@@ -91,7 +92,7 @@ def test_flash_forward_declines_unsupported_shapes():
     i = torch.ones(4, dtype=torch.int32, device="cuda")
     ok = (ptr(t), ptr(t), ptr(t), F16, ptr(f), ptr(i), ptr(t), ptr(f))
     assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 8, 64, 64, 64, 512, 64, 512, stream()) == -1      # head size 64
-    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 6, 128, 128, 128, 768, 128, 768, stream()) == -1  # tokens % 4
+    assert lib.br_hip_flash_attn_fwd(*ok, 1, 1, 8, 128, 132, 128, 1056, 128, 1024, stream()) == -1  # row stride % 8
     assert lib.br_hip_flash_attn_fwd(ptr(t), ptr(t), ptr(t), hip.F32, ptr(f), ptr(i), ptr(t), ptr(f), 1, 1, 8, 128,
                                      128, 128, 1024, 128, 1024, stream()) == -1
     assert lib.br_hip_flash_attn_fwd(None, ptr(t), ptr(t), F16, ptr(f), ptr(i), ptr(t), ptr(f), 1, 1, 8, 128, 128,
@@ -106,6 +107,7 @@ def test_flash_forward_declines_unsupported_shapes():
     (2, 3, 200, (200, 1)),
     (2, 2, 132, (0, 77)),
     (1, 1, 4, (3,)),
+    (1, 2, 37, (30,)),            # odd token count
 ])
 def test_flash_backward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype):
     """dq, dk, dv against the oracle's attention-backward, softmax-backward and
