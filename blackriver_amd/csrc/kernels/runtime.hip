@@ -7,6 +7,26 @@
 
 using namespace brk;
 
+namespace {
+
+// Byte fill as a kernel rather than hipMemsetAsync, so that a caller may record
+// it into a HIP graph like any other launch: 16-byte stores over the aligned
+// middle, single bytes at both ends.
+__global__ __launch_bounds__(256) void memset_kernel(unsigned char* dst, unsigned char value, size_t bytes) {
+    const size_t head = (16 - (reinterpret_cast<uintptr_t>(dst) & 15)) & 15;
+    const size_t lead = head < bytes ? head : bytes;
+    const size_t vecs = (bytes - lead) / 16;
+    const size_t tid = (size_t)blockIdx.x * 256 + threadIdx.x, stride = (size_t)gridDim.x * 256;
+    const unsigned w = value * 0x01010101u;
+    uint4* mid = reinterpret_cast<uint4*>(dst + lead);
+    for (size_t i = tid; i < vecs; i += stride) mid[i] = make_uint4(w, w, w, w);
+    const size_t tail0 = lead + vecs * 16;
+    for (size_t i = tid; i < lead; i += stride) dst[i] = value;
+    for (size_t i = tail0 + tid; i < bytes; i += stride) dst[i] = value;
+}
+
+}  // namespace
+
 extern "C" {
 
 int br_hip_device_count(int* count) {
@@ -122,7 +142,10 @@ int br_hip_memcpy_d2d(void* dst, const void* src, size_t bytes, br_stream_t stre
 
 int br_hip_memset(void* dst, int byte_value, size_t bytes, br_stream_t stream) {
     if (bytes == 0) return BR_OK;
-    BR_HIP_TRY(hipMemsetAsync(dst, byte_value, bytes, as_stream(stream)));
+    if (!dst) return BR_ERR_OUTPUT;
+    memset_kernel<<<grid_for((int64_t)(bytes / 16 + 1), 256), 256, 0, as_stream(stream)>>>(
+        static_cast<unsigned char*>(dst), (unsigned char)byte_value, bytes);
+    BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }
 

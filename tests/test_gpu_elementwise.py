@@ -316,3 +316,14 @@ def test_adamw_rejects_bad_arguments():
     assert lib.br_hip_adamw(None, F32, None, ptr(t), ptr(t), ptr(t), *args, 1, stream()) == -3
     assert lib.br_hip_adamw(ptr(t), I32, None, ptr(t), ptr(t), ptr(t), *args, 1, stream()) == -1
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("offset,nbytes", [(0, 1 << 20), (3, 1000), (5, 7), (16, 4096 + 9), (1, 0)])
+def test_memset_fills_exactly_the_requested_bytes(offset, nbytes):
+    """br_hip_memset is a fill kernel (16-byte stores over the aligned middle,
+    single bytes at the ends): every requested byte is set, none around it."""
+    buf = torch.full((nbytes + 64,), 0x11, dtype=torch.uint8, device="cuda")
+    call("br_hip_memset", ctypes.c_void_p(buf.data_ptr() + offset), 0xAB, nbytes, stream())
+    got = host(buf)
+    assert np.all(got[offset:offset + nbytes] == 0xAB)
+    assert np.all(got[:offset] == 0x11) and np.all(got[offset + nbytes:] == 0x11)
