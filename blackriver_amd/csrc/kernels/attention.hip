@@ -101,39 +101,26 @@ struct TileLoader {
     }
 };
 
-// A operand, rows of the tile as MFMA rows, d as the k index: rows r0 + lane%32,
-// d = 16 * ks + 8 * (lane / 32) .. + 7.
-__device__ __forceinline__ u32x4 frag_rows(const lds_byte* tile, int r0, int ks, int lane) {
-    const int r = r0 + (lane & 31);
-    return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(tile + slot(r, ks * 2 + (lane >> 5)));
-}
-
-// A / B operand with d as the MFMA row (or column) index and tile rows as the
-// k index: lane gets d = d0 + 16 * ((lane >> 4) & 1) + lane % 16 and the eight
-// tile rows  ra + 0..3  and  rb + 0..3  (ra, rb multiples of 4, per lane half).
-__device__ __forceinline__ u32x4 frag_cols(const lds_byte* tile, int d0, int ra, int rb, int lane) {
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    const int i = lane & 15;
-    const int d = d0 + ((lane >> 4) & 1) * 16 + (i & 3) * 4;
-    const int ja = ra + (i >> 2), jb = rb + (i >> 2);
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + slot(ja, d >> 3) + (d & 7) * 2));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + slot(jb, d >> 3) + (d & 7) * 2));
-    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-    return mk4(l2.x, l2.y, h2.x, h2.y);
-}
-
-// The same two reads with every lane-dependent part of the address computed
-// once (FragOffsets) and everything else a compile-time constant, so that the
-// reads inside the tile loops need no address arithmetic at all.
+// MFMA operand fragments of a tile image.  Every lane-dependent part of an
+// address is computed once (constructor); inside the tile loops a read is that
+// per-lane offset plus compile-time constants, i.e. no address arithmetic.
+//   frag_rows: tile rows as MFMA rows (or columns), d as the k index: row
+//       r0 + lane % 32, d = 16 * ks + 8 * (lane / 32) .. + 7; one 128-bit read.
+//   frag_cols: d as the MFMA row (or column) index, tile rows as the k index:
+//       d = 32 * db + lane % 32 and the eight tile rows r16 + 4 * half + 0..3 and
+//       + 8 (half = lane / 32) -- the row order an accumulator block holds, so
+//       that probabilities / score gradients go from accumulators straight into
+//       the other operand; two transposing 64-bit reads.
 struct FragOffsets {
-    unsigned rows[8];            // frag_rows(tile, 0, ks, lane) - tile
-    unsigned cols_lo[4], cols_hi[4];  // frag_cols(tile, 32 * db, 4 * half, 4 * half + 8, lane) - tile
+    unsigned rows[8];
+    unsigned cols_lo[4], cols_hi[4];
     __device__ __forceinline__ explicit FragOffsets(int lane) {
         const int i = lane & 15, half = lane >> 5;
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) rows[ks] = slot(lane & 31, ks * 2 + half);
 #pragma unroll
         for (int db = 0; db < 4; db++) {
+            // a group of 16 lanes reads 4 tile rows (i >> 2) x 16 d; lane i receives d column i
             const int d = db * 32 + ((lane >> 4) & 1) * 16 + (i & 3) * 4;
             const int ja = half * 4 + (i >> 2);
             cols_lo[db] = slot(ja, d >> 3) + (d & 7) * 2;
@@ -144,7 +131,7 @@ struct FragOffsets {
     __device__ __forceinline__ u32x4 frag_rows(const lds_byte* lds, int tile, int r0, int ks) const {
         return *reinterpret_cast<const __attribute__((address_space(3))) u32x4*>(lds + rows[ks] + (tile + r0 * 256));
     }
-    // tile rows r16 + 4 * half + 0..3 and + 8 (r16 a multiple of 16), d block db
+    // r16 a multiple of 16
     __device__ __forceinline__ u32x4 frag_cols(const lds_byte* lds, int tile, int db, int r16) const {
         typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lds + cols_lo[db] + (tile + r16 * 256)));
