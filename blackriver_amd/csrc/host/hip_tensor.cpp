@@ -92,6 +92,18 @@ Operand shared_operand(const void* p, int dtype, int64_t items, int compute) {
     return {dst, native};
 }
 
+// The two products of a linear layer's backward once the gradient dy[n,out] is
+// available in the products' type: weight_g[out,in] = dy^T . x, then
+// x_g[n,in] = dy . W (in that order: x_g may overwrite x).
+int linear_backward_products(const Operand& dy, const tensor_t& x, const tensor_t& weight, const tensor_t& x_g,
+                             const tensor_t& weight_g, int64_t n, int64_t in, int64_t out, int compute) {
+    int rc = product(1, 0, out, in, n, 1.0f, dy.ptr, dy.dtype, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
+                     code(weight_g), in, 0, nullptr, 1, compute);
+    if (rc != BR_OK) return rc;
+    return product(0, 0, n, in, out, 1.0f, dy.ptr, dy.dtype, out, 0, weight->data(), code(weight), in, 0, 0,
+                   x_g->data(), code(x_g), in, 0, nullptr, 1, compute);
+}
+
 // fp32 device pointer to a bias vector, converting 16-bit storage on the fly
 // into workspace tail slot `slot` (each slot 1 MiB).
 const float* bias_f32(const tensor_t& b, int slot) {
@@ -565,12 +577,7 @@ ComputingReturn HIPTensor<DT>::op_linear_backward(tensor_t self, tensor_t x, ten
         BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, ws, need, stream()));
         dy = shared_operand(mem_, (int)DT, n * out, compute);
     }
-    // weight_g[out,in] = dy^T . x
-    BR_OP(product(1, 0, out, in, n, 1.0f, dy.ptr, dy.dtype, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
-                  code(weight_g), in, 0, nullptr, 1, compute));
-    // x_g[n,in] = dy . W
-    BR_OP(product(0, 0, n, in, out, 1.0f, dy.ptr, dy.dtype, out, 0, weight->data(), code(weight), in, 0, 0,
-                  x_g->data(), code(x_g), in, 0, nullptr, 1, compute));
+    BR_OP(linear_backward_products(dy, x, weight, x_g, weight_g, n, in, out, compute));
     return OP_OK;
 }
 
@@ -678,6 +685,40 @@ ComputingReturn HIPTensor<DT>::op_qk_backward(tensor_t self, tensor_t q, tensor_
     BR_OP(product(1, 0, t, hd, t, alpha, ds.ptr, ds.dtype, t, t * t, q->data(), code(q), hd, t * hd, 0, k_g->data(),
                   code(k_g), hd, t * hd, nullptr, bh, compute));
     return OP_OK;
+}
+
+ComputingReturn hip_gelu_linear_backward(const tensor_t& dy, const tensor_t& u, const tensor_t& du, const tensor_t& x,
+                                         const tensor_t& weight, const tensor_t& bias, const tensor_t& x_g,
+                                         const tensor_t& weight_g, const tensor_t& bias_g) {
+    bool fast = dev_f32(dy) && dev_f32(u) && dev_f32(du) && dev(x) && dev(weight) && dev(x_g) && dev(weight_g) &&
+                dev_f32(bias_g) && du->shape().dim() == 3 && x->shape().dim() == 3 && u->items() == dy->items() &&
+                du->items() == dy->items();
+    if (fast) {
+        const int64_t n = (int64_t)(du->shape()[0] * du->shape()[1]);
+        const int64_t out = (int64_t)du->shape()[2], in = (int64_t)x->shape()[2];
+        const int compute = pick_compute({du, x, weight});
+        fast = compute != BR_GEMM_F32 && out % 8 == 0 && (int64_t)x->items() == n * in &&
+               (int64_t)weight->items() == out * in && (int64_t)x_g->items() == n * in &&
+               (int64_t)weight_g->items() == out * in && (int64_t)bias_g->items() == out;
+        if (fast) {
+            const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
+            const size_t need = br_hip_colsum_workspace(n, out);
+            void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
+            void* dy16 = ComputingContext::gemm_staging(1, (size_t)(n * out) * 2);
+            const int rc = br_hip_gelu_bwd_colsum_cast(
+                static_cast<const float*>(dy->data()), static_cast<const float*>(u->data()),
+                static_cast<float*>(du->data()), static_cast<float*>(bias_g->data()), dy16, native, n, out, ws, need,
+                stream());
+            if (rc != BR_ERR_TODO) {
+                BR_OP(rc);
+                BR_OP(linear_backward_products(Operand{dy16, native}, x, weight, x_g, weight_g, n, in, out, compute));
+                return OP_OK;
+            }
+        }
+    }
+    ComputingReturn r = dy->op_gelu_backward(dy, u, du);
+    if (r != OP_OK) return r;
+    return du->op_linear_backward(du, x, weight, bias, x_g, weight_g, bias_g);
 }
 
 ComputingReturn hip_linear_accumulate(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& y) {

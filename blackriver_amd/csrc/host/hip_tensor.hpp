@@ -71,6 +71,12 @@ private:
     const bool owner_;
 };
 
+// op_gelu_backward(dy, u, du) followed by op_linear_backward(du, x, ...): with a
+// 16-bit MFMA type one pass produces du, its 16-bit copy and the bias gradient
+// (same bits as the two operators), then the two products run.
+ComputingReturn hip_gelu_linear_backward(const tensor_t& dy, const tensor_t& u, const tensor_t& du, const tensor_t& x,
+                                         const tensor_t& weight, const tensor_t& bias, const tensor_t& x_g,
+                                         const tensor_t& weight_g, const tensor_t& bias_g);
 // y += x . w^T + bias: op_linear (cuda_tensor.cpp:146-193) followed by
 // op_add(y, ., y) with the addition done in the product's epilogue; the sum is
 // formed from the same fp32 values, so the bits equal the two operators'.

@@ -337,6 +337,19 @@ BR_WORD(FlashAttnQkvBackward,
 
 // Two operator pairs of the model scripts with the addition folded into the
 // producing kernel (same bits as the pair; no counterpart word in the reference):
+// ( dy u du   du' x w b x_g w_g b_g -- )  `op.gelu_backward` followed by the
+// `op.linear_backward` of the layer below; fused when du' is du
+BR_WORD(GeluLinearBackward,
+    Tensors<7> l(stack);
+    Tensors<3> g(stack);
+    if (l[0]->data() == g[2]->data() && l[0]->items() == g[2]->items()) {
+        op_check_word(hip_gelu_linear_backward(g[0], g[1], g[2], l[1], l[2], l[3], l[4], l[5], l[6]),
+                      "op.gelu_backward + op.linear_backward");
+    } else {
+        g[0]->op_gelu_backward(g[0], g[1], g[2]);
+        l[0]->op_linear_backward(l[0], l[1], l[2], l[3], l[4], l[5], l[6]);
+    }
+)
 // ( x w b y -- )   y += x . w^T + b          `op.linear` into a temporary + `op.add`
 BR_WORD(LinearAdd,
     Tensors<4> a(stack);
@@ -434,6 +447,7 @@ void load_nn_words(Enviroment& env) {
         {"op.softmax_backward", SoftmaxBackward::creator},
         {"op.softmax_attn_backward", SoftmaxAttnBackward::creator},
         {"op.qk_backward", QueryKeyBackward::creator},
+        {"op.gelu_linear_backward", GeluLinearBackward::creator},
         {"op.linear_add", LinearAdd::creator},
         {"op.layernorm_backward_add", LayernormBackwardAdd::creator},
         {"op.flash_attn", FlashAttn::creator},
@@ -448,6 +462,7 @@ void load_nn_words(Enviroment& env) {
     env.insert_fusion({"op.add", "op.add", "op.softmax", "op.copy"}, "op.add_add_softmax_copy");
     env.insert_fusion({"op.add", "op.add", "op.softmax"}, "op.add_add_softmax");
     env.insert_fusion({"op.layernorm", "op.copy"}, "op.layernorm_copy");
+    env.insert_fusion({"op.gelu_backward", "op.linear_backward"}, "op.gelu_linear_backward");
 }
 
 }  // namespace br

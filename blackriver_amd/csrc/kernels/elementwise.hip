@@ -513,6 +513,57 @@ __global__ __launch_bounds__(kBlock) void colsum_cast_partial(const float* __res
     for (int j = 0; j < 4; j++) partial[(int64_t)blockIdx.y * cols + col + j] = acc[j];
 }
 
+// The same pass with x produced on the fly: x = dy * gelu'(u), the GELU
+// backward whose result is the gradient of the linear layer below it.  Writes
+// the fp32 gradient (dx may be u's or dy's own buffer), its 16-bit copy and
+// the column-sum partials; dx is rounded to fp32 before it is summed and
+// converted, so all three equal what the separate kernels produce.
+template <typename D>
+__global__ __launch_bounds__(kBlock) void gelu_bwd_colsum_cast_partial(const float* dy, const float* u, float* dx,
+                                                                        float* __restrict__ partial,
+                                                                        D* __restrict__ dx16, int64_t rows,
+                                                                        int64_t cols, int rows_per_block) {
+    const int64_t col = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * 4;
+    if (col >= cols) return;
+    const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
+    const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    auto emit = [&](int64_t r, const float (&g)[4], const float (&x)[4]) {
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            v[j] = g[j] * gelu_grad_one(x[j]);
+            asm volatile("" : "+v"(v[j]));
+            acc[j] += v[j];
+        }
+        VecIO<float, 4>::store(dx + r * cols + col, v);
+        const unsigned lo = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[0])) |
+                            ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[1])) << 16);
+        const unsigned hi = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[2])) |
+                            ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[3])) << 16);
+        *reinterpret_cast<uint2*>(dx16 + r * cols + col) = make_uint2(lo, hi);
+    };
+    int64_t r = r0;
+    for (; r + 2 <= r1; r += 2) {
+        float g[2][4], x[2][4];
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            VecIO<float, 4>::load(dy + (r + k) * cols + col, g[k]);
+            VecIO<float, 4>::load(u + (r + k) * cols + col, x[k]);
+        }
+#pragma unroll
+        for (int k = 0; k < 2; k++) emit(r + k, g[k], x[k]);
+    }
+    for (; r < r1; r++) {
+        float g[4], x[4];
+        VecIO<float, 4>::load(dy + r * cols + col, g);
+        VecIO<float, 4>::load(u + r * cols + col, x);
+        emit(r, g, x);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) partial[(int64_t)blockIdx.y * cols + col + j] = acc[j];
+}
+
 // Stage 2 for cols % 4 == 0: 1024 threads = 16 column quads x 64 slices of
 // groups, every load of a workgroup in flight at once; slices are combined in
 // LDS in a fixed order.
@@ -1054,6 +1105,33 @@ int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int
         colsum_cast_partial<__half><<<grid, kBlock, 0, st>>>(x, partial, (__half*)x16, rows, cols, rpb);
     else
         colsum_cast_partial<__hip_bfloat16><<<grid, kBlock, 0, st>>>(x, partial, (__hip_bfloat16*)x16, rows, cols, rpb);
+    BR_HIP_LAUNCH_CHECK();
+    return colsum_finish(partial, out, groups, cols, st);
+}
+
+int br_hip_gelu_bwd_colsum_cast(const float* dy, const float* x, float* dx, float* out, void* dx16, int dx16_dtype,
+                                int64_t rows, int64_t cols, void* workspace, size_t workspace_bytes,
+                                br_stream_t stream) {
+    if (rows <= 0 || cols <= 0) return BR_ERR_ATTR;
+    if (!dy || !x) return BR_ERR_INPUT;
+    if (!dx || !out || !dx16) return BR_ERR_OUTPUT;
+    if (dx16_dtype != BR_F16 && dx16_dtype != BR_BF16) return BR_ERR_TODO;
+    if (cols % 4 != 0 || !aligned16(dy) || !aligned16(x) || !aligned16(dx) ||
+        (reinterpret_cast<uintptr_t>(dx16) & 7u) != 0)
+        return BR_ERR_TODO;
+    if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
+    hipStream_t st = as_stream(stream);
+    float* partial = (float*)workspace;
+    // same strips as br_hip_colsum_cast, hence the same summation order
+    const int64_t blocks_x = (cols / 4 + kBlock - 1) / kBlock;
+    const int rpb = colsum_vec_rows_per_block(rows, blocks_x);
+    const int groups = (int)((rows + rpb - 1) / rpb);
+    dim3 grid((unsigned)blocks_x, (unsigned)groups);
+    if (dx16_dtype == BR_F16)
+        gelu_bwd_colsum_cast_partial<__half><<<grid, kBlock, 0, st>>>(dy, x, dx, partial, (__half*)dx16, rows, cols, rpb);
+    else
+        gelu_bwd_colsum_cast_partial<__hip_bfloat16><<<grid, kBlock, 0, st>>>(dy, x, dx, partial,
+                                                                             (__hip_bfloat16*)dx16, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
     return colsum_finish(partial, out, groups, cols, st);
 }

@@ -57,6 +57,7 @@ SIGNATURES = {
     "br_hip_colsum_workspace": (_sz, [_i64, _i64]),
     "br_hip_colsum_cast": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp, _sz, _vp]),
     "br_hip_colsum": (_int, [_vp, _int, _vp, _i64, _i64, _vp, _sz, _vp]),
+    "br_hip_gelu_bwd_colsum_cast": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _vp, _sz, _vp]),
     "br_hip_layernorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "br_hip_layernorm_fwd_copy16": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _f32, _vp]),
     "br_hip_layernorm_bwd_workspace": (_sz, [_i64, _i64]),

@@ -136,6 +136,17 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
 int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int64_t rows, int64_t cols,
                        void* workspace, size_t workspace_bytes, br_stream_t stream);
 
+/* br_hip_gelu_bwd (fp32) and br_hip_colsum_cast in one pass: dx = dy * gelu'(x)
+ * is written as fp32 (dx may be x's or dy's own buffer), as a 16-bit copy dx16
+ * and column-summed into out -- `op.gelu_backward` followed by the head of the
+ * `op.linear_backward` below it (bloomz-7b/train.words:200-202; gelu.cu:61-85,
+ * cuda_tensor.cpp:730-760).  All three results are bit for bit those of the two
+ * separate entries.  BR_ERR_TODO unless cols % 4 == 0 and 16-byte aligned
+ * operands; workspace as for br_hip_colsum. */
+int br_hip_gelu_bwd_colsum_cast(const float* dy, const float* x, float* dx, float* out, void* dx16,
+                                int dx16_dtype, int64_t rows, int64_t cols, void* workspace,
+                                size_t workspace_bytes, br_stream_t stream);
+
 /* ---- LayerNorm --------------------------------------------------------- */
 /* kernels::launch_layer_norm_float, kernels/normalize_kernels.cu:87-102
  * (declared kernels/kernels.h:24), called at cuda_tensor.cpp:236-255.  var receives sigma^2 + eps; mean and

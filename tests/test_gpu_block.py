@@ -358,3 +358,43 @@ def test_linear_add_and_layernorm_backward_add_words_equal_the_operator_pairs(ru
             assert np.array_equal(env.read("dgam2"), env.read("dgam")) and np.array_equal(env.read("dbet2"), env.read("dbet"))
         finally:
             env.close()
+
+
+@pytest.mark.parametrize("mode", ["f16", "f32"])
+def test_fused_gelu_backward_linear_backward_equals_the_two_words(runtime, mode):
+    """The fusion pass turns `op.gelu_backward op.linear_backward` (the pair of
+    bloomz-7b/train.words:200-202) into one word; run as one program (fused)
+    and as two programs (not fused) it must leave identical tensors, in the
+    16-bit product mode (fused kernel) and in fp32 mode (the word's fallback)."""
+    rng = np.random.default_rng(13)
+    b, t, hidden = 2, 24, 128
+    env = host.Env(1)
+    try:
+        env.execute("'%s' op.gemm_precision" % mode)
+        wdt = "f16" if mode == "f16" else "float"
+        env.execute("%d %d %d 3 'cuda' 'float' op.create 'dy' !  %d %d %d 3 'cuda' 'float' op.create 'u' !"
+                    % (b, t, 4 * hidden, b, t, 4 * hidden))
+        env.execute("%d %d %d 3 'cuda' 'float' op.create 'x' !  %d %d %d 3 'cuda' 'float' op.create 'xg' !"
+                    % (b, t, hidden, b, t, hidden))
+        env.execute("%d %d 2 'cuda' '%s' op.create 'w' !  %d %d 2 'cuda' 'float' op.create 'wg' !"
+                    % (4 * hidden, hidden, wdt, 4 * hidden, hidden))
+        env.execute("%d 1 'cuda' 'float' op.create 'bias' !  %d 1 'cuda' 'float' op.create 'bg' !"
+                    % (4 * hidden, 4 * hidden))
+        u0 = (1.5 * rng.standard_normal((b, t, 4 * hidden))).astype(np.float32)
+        env.write("dy", rng.standard_normal((b, t, 4 * hidden)).astype(np.float32))
+        env.write("x", rng.standard_normal((b, t, hidden)).astype(np.float32))
+        env.write("w", (0.05 * rng.standard_normal((4 * hidden, hidden))).astype(np.float32))
+        gelu = "'dy' @ 'u' @ 'u' @ op.gelu_backward"
+        lin = "'u' @ 'x' @ 'w' @ 'bias' @ 'xg' @ 'wg' @ 'bg' @ op.linear_backward"
+        assert "W:op.gelu_linear_backward" in env.disassemble(gelu + "  " + lin, fused=True)
+        env.write("u", u0)
+        env.execute(gelu)
+        env.execute(lin)
+        want = {n: env.read(n) for n in ("u", "xg", "wg", "bg")}
+        env.write("u", u0)
+        env.execute("'xg' @ op.zero 'wg' @ op.zero 'bg' @ op.zero")
+        env.execute(gelu + "  " + lin)
+        for n, v in want.items():
+            assert np.array_equal(env.read(n), v), (mode, n)
+    finally:
+        env.close()

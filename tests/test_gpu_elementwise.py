@@ -327,3 +327,34 @@ def test_memset_fills_exactly_the_requested_bytes(offset, nbytes):
     got = host(buf)
     assert np.all(got[offset:offset + nbytes] == 0xAB)
     assert np.all(got[:offset] == 0x11) and np.all(got[offset + nbytes:] == 0x11)
+
+
+@pytest.mark.parametrize("dtype,tdtype", [(F16, torch.float16), (BF16, torch.bfloat16)])
+@pytest.mark.parametrize("rows,cols", [(2048, 16384), (37, 64), (5, 1000)])
+def test_gelu_bwd_colsum_cast_equals_the_separate_kernels(rows, cols, dtype, tdtype):
+    """One pass producing the GELU gradient, its 16-bit copy and its column
+    sums: each bit for bit what br_hip_gelu_bwd followed by br_hip_colsum_cast
+    gives, also in place on x."""
+    print("case rows=%d cols=%d dtype=%d" % (rows, cols, dtype), flush=True)
+    rng = np.random.default_rng(23)
+    x = (1.5 * rng.standard_normal((rows, cols))).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    d_x, d_dy = dev(x), dev(dy)
+    n = rows * cols
+    dx_sep = empty((rows, cols))
+    call("br_hip_gelu_bwd", ptr(d_dy), ptr(d_x), ptr(dx_sep), F32, n, stream())
+    ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
+    sums_sep, x16_sep = empty(cols), empty((rows, cols), tdtype)
+    call("br_hip_colsum_cast", ptr(dx_sep), ptr(sums_sep), ptr(x16_sep), dtype, rows, cols, ptr(ws), ws.numel(), stream())
+    for in_place in (False, True):
+        d_u = dev(x)
+        dx = d_u if in_place else empty((rows, cols))
+        sums, x16 = empty(cols), empty((rows, cols), tdtype)
+        call("br_hip_gelu_bwd_colsum_cast", ptr(d_dy), ptr(d_u), ptr(dx), ptr(sums), ptr(x16), dtype, rows, cols,
+             ptr(ws), ws.numel(), stream())
+        assert torch.equal(dx, dx_sep), in_place
+        assert torch.equal(x16.view(torch.int16), x16_sep.view(torch.int16)), in_place
+        assert torch.equal(sums, sums_sep), in_place
+    assert hip.load().br_hip_gelu_bwd_colsum_cast(ptr(d_dy), ptr(d_x), ptr(dx_sep), ptr(sums_sep), ptr(x16_sep), dtype,
+                                                  4, 1001, ptr(ws), ws.numel(), stream()) == -1
+    torch.cuda.synchronize()
