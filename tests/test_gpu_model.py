@@ -6,6 +6,7 @@ the GPU by the C++ driver, compared with the CPU oracle's composition
   fp32 mode: fp32 weights, fp32 MFMA products; bound 2e-4 (a chain of
              3 x ~20 fp32 operators plus the head, each within 1e-5)
   f16 mode:  fp16 weights, fp16 MFMA products, fp32 accumulation; bound 2e-2
+  bf16 mode: bf16 weights and products; bound 1e-1 (8 times coarser rounding)
 """
 import numpy as np
 import pytest
@@ -24,9 +25,9 @@ MODEL_NAMES = ["word_embeddings.weight", "word_embeddings_layernorm.weight", "wo
 
 def build(mode, layers, batch, tokens, hidden, heads, vocab, seed):
     rng = np.random.default_rng(seed)
-    f16 = mode == "f16"
-    model = host.BloomModel(layers, batch, tokens, hidden, heads, vocab, 1e-5, "f16" if f16 else "float",
-                            "f16" if f16 else "f32")
+    wdtype = {"f16": "f16", "bf16": "bf16"}.get(mode, "float")
+    model = host.BloomModel(layers, batch, tokens, hidden, heads, vocab, 1e-5, wdtype,
+                            wdtype if wdtype != "float" else "f32")
     model.init(seed, 0.05)
     # LayerNorm parameters and biases away from their 1 / 0 defaults
     for i in range(1, layers + 1):
@@ -50,11 +51,14 @@ def build(mode, layers, batch, tokens, hidden, heads, vocab, seed):
     ("fp32", 3, 2, 32, 256, 4, 1024),
     ("f16", 2, 2, 64, 512, 8, 2048),
     ("f16", 2, 2, 64, 512, 4, 2048),      # head size 128: attention runs as the fused kernels
+    ("bf16", 2, 2, 64, 512, 4, 2048),     # the same in bf16 (8-bit mantissa; see the bound below)
 ])
 def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden, heads, vocab):
     print("case %s layers=%d batch=%d tokens=%d hidden=%d" % (mode, layers, batch, tokens, hidden), flush=True)
     model, model_w, layer_ws, ids, mask = build(mode, layers, batch, tokens, hidden, heads, vocab, seed=7)
-    tol = 2e-4 if mode == "fp32" else 2e-2
+    # bf16: one block holds 6e-2 (tests/test_gpu_block.py); two blocks, the head and the tied
+    # table's gradient (a sum of two bf16-product results) compound to just under 1e-1
+    tol = {"fp32": 2e-4, "f16": 2e-2, "bf16": 1e-1}[mode]
     try:
         # different initial matrices per block (a seed slip would make them equal)
         assert not np.array_equal(layer_ws[0]["dense.weight"], layer_ws[1]["dense.weight"])
