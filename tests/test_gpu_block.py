@@ -398,3 +398,26 @@ def test_fused_gelu_backward_linear_backward_equals_the_two_words(runtime, mode)
             assert np.array_equal(env.read(n), v), (mode, n)
     finally:
         env.close()
+
+
+def test_fused_attention_follows_the_mask_tables_prefix_rule(runtime):
+    """A mask with a hole: the reference's table closes every key from the
+    first zero on (train_bloom.cpp:73-90), so `bloom.valid` must report the
+    length of the leading run of non-zeros, and the fused path must match the
+    operator chain that reads the table."""
+    hidden, heads, batch, tokens = 256, 2, 2, 32
+    env, w, x, dy, mask, _ = setup_block(runtime, hidden, heads, batch, tokens, "f16")
+    mask = np.ones((batch, tokens), np.int32)
+    mask[0, 10] = 0          # a hole: keys 10.. are closed although 11.. are non-zero
+    mask[1, 0] = 0           # nothing open at all: uniform probabilities
+    env.write("mask_", mask)
+    env.execute("create_operand_buffers create_flash_buffers prepare_batch_flash")
+    assert list(env.read("xvalid").view(np.int32)[:batch]) == [10, 0]
+    env.execute("layer_forward_flash op.sync")
+    flash = env.read("xa")
+    saved = blk.layer_forward(w, x, orc.alibi(heads, tokens), orc.xmask(mask), heads, 1e-5)
+    assert_close(flash, saved["xa"], 2e-2, "block output against the oracle")
+    env.write("xinput", x)
+    env.execute("layer_forward_mixed op.sync")
+    assert_close(flash, env.read("xa"), 2e-2, "block output against the operator chain")
+    env.close()
