@@ -421,3 +421,48 @@ def test_fused_attention_follows_the_mask_tables_prefix_rule(runtime):
     env.execute("layer_forward_mixed op.sync")
     assert_close(flash, env.read("xa"), 2e-2, "block output against the operator chain")
     env.close()
+
+
+def test_flash_attention_words_on_separate_and_packed_projections_agree(runtime):
+    """`op.flash_attn` / `op.flash_attn_backward` take q, k, v as three
+    [B, T, heads, 128] tensors, the `_qkv` forms one packed [B, T, 3H] tensor
+    read through strides: same kernels, so the same bits."""
+    rng = np.random.default_rng(17)
+    b, t, nh, hd = 2, 48, 2, 128
+    h = nh * hd
+    env = host.Env(1)
+    try:
+        for n in ("q", "k", "v", "o", "o2", "g"):
+            env.execute("%d %d %d %d 4 'cuda' 'f16' op.create '%s' !" % (b, t, nh, hd, n))
+        env.execute("%d %d %d 3 'cuda' 'f16' op.create 'qkv' !" % (b, t, 3 * h))
+        env.execute("%d %d %d 3 'cuda' 'float' op.create 'dqkv' !" % (b, t, 3 * h))
+        for n in ("dq", "dk", "dv"):
+            env.execute("%d %d %d %d 4 'cuda' 'float' op.create '%s' !" % (b, t, nh, hd, n))
+        env.execute("%d %d %d 3 'cuda' 'float' op.create 'lse' !  %d %d %d 3 'cuda' 'float' op.create 'lse2' !"
+                    % (b, nh, t, b, nh, t))
+        env.execute("1 %d 1 %d 4 'cuda' 'float' op.create 'alibi' !  %d 1 'cuda' 'float' op.create 'valid' !" % (nh, t, b))
+        env.execute("%d %d 2 'cpu' 'int' op.create 'mask' !" % (b, 1024 // b))   # cpu tensors come in 1024-item granules
+        q, k, v, g = (rng.standard_normal((b, t, nh, hd)).astype(np.float16).astype(np.float32) for _ in range(4))
+        for n, a in (("q", q), ("k", k), ("v", v), ("g", g)):
+            env.write(n, a)
+        env.write("qkv", np.concatenate([q.reshape(b, t, h), k.reshape(b, t, h), v.reshape(b, t, h)], axis=2))
+        m = np.zeros((b, 1024 // b), np.int32)
+        m[0, :t] = 1
+        m[1, :t - 7] = 1
+        env.execute("'alibi' @ bloom.alibi")
+        # bloom.valid reads [batch, tokens] rows of the mask it is given: a [B, T] view of the granule-sized tensor
+        env.execute("'mask' @ 0 %d %d 2 op.view 'mask_bt' !" % (b, t))
+        env.write("mask_bt", np.ascontiguousarray(m[:, :t]))
+        env.execute("'mask_bt' @ 'valid' @ bloom.valid")
+        assert list(env.read("valid").view(np.int32)[:b]) == [t, t - 7]
+        env.execute("'q' @ 'k' @ 'v' @ 'alibi' @ 'valid' @ 'o' @ 'lse' @ op.flash_attn")
+        env.execute("'qkv' @ 'alibi' @ 'valid' @ 'o2' @ 'lse2' @ op.flash_attn_qkv")
+        assert np.array_equal(env.read("o"), env.read("o2")) and np.array_equal(env.read("lse"), env.read("lse2"))
+        assert np.all(np.isfinite(env.read("o"))) and np.any(env.read("o") != 0)
+        env.execute("'q' @ 'k' @ 'v' @ 'o' @ 'g' @ 'alibi' @ 'valid' @ 'lse' @ 'dq' @ 'dk' @ 'dv' @ op.flash_attn_backward")
+        env.execute("'qkv' @ 'o' @ 'g' @ 'alibi' @ 'valid' @ 'lse' @ 'dqkv' @ op.flash_attn_qkv_backward")
+        packed = env.read("dqkv")
+        for i, n in enumerate(("dq", "dk", "dv")):
+            assert np.array_equal(packed[:, :, i * h:(i + 1) * h], env.read(n).reshape(b, t, h)), n
+    finally:
+        env.close()
