@@ -478,23 +478,35 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
                           code(lm_head), hidden, 0, 0, logits, BR_F32, vocab, 0, nullptr, 1, compute));
         BR_OP(br_hip_logsoftmax_nll_fwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, d_logp + r0, d_result, rows,
                                         vocab, stream()));
-        // dlogits: written as fp16 straight away when the products run in fp16
-        // (the same rounding the GEMM would apply to an fp32 copy), else fp32
-        // in place and converted once for the two products below
+        // dlogits.  With fp32 products it is scaled by 1/count in place, as the
+        // reference does.  With 16-bit products the stored operand leaves 1/count
+        // out (p/count would fall below fp16's smallest subnormal at a real
+        // vocabulary size) and, for fp16, carries an exact factor 2^14 that lifts
+        // probabilities down to 4e-12 into range (|softmax - onehot| <= 1, so no
+        // overflow); both factors go into the products' alpha.
         Operand dl{logits, BR_F32};
-        if (compute == BR_GEMM_F16 && (rows * vocab) % 8 == 0) {
-            void* dl16 = ComputingContext::gemm_staging(1, (size_t)(rows * vocab) * 2);
-            BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, dl16, BR_F16, scale, rows,
-                                            vocab, stream()));
-            dl = Operand{dl16, BR_F16};
-        } else {
+        float alpha = 1.0f;
+        if (compute == BR_GEMM_F32) {
             BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, logits, BR_F32, scale,
                                             rows, vocab, stream()));
-            dl = shared_operand(logits, BR_F32, rows * vocab, compute);
+        } else {
+            const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
+            const float lift = compute == BR_GEMM_F16 ? 16384.0f : 1.0f;
+            alpha = scale / lift;
+            if ((rows * vocab) % 8 == 0) {
+                void* dl16 = ComputingContext::gemm_staging(1, (size_t)(rows * vocab) * 2);
+                BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, dl16, native, lift,
+                                                rows, vocab, stream()));
+                dl = Operand{dl16, native};
+            } else {
+                BR_OP(br_hip_logsoftmax_nll_bwd(logits, d_labels + r0, d_keep + r0, d_lse + r0, logits, BR_F32, lift,
+                                                rows, vocab, stream()));
+                dl = shared_operand(logits, BR_F32, rows * vocab, compute);
+            }
         }
-        BR_OP(product(0, 0, rows, hidden, vocab, 1.0f, dl.ptr, dl.dtype, vocab, 0, lm_head->data(), code(lm_head),
+        BR_OP(product(0, 0, rows, hidden, vocab, alpha, dl.ptr, dl.dtype, vocab, 0, lm_head->data(), code(lm_head),
                       hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute));
-        BR_OP(product(1, 0, vocab, hidden, rows, 1.0f, dl.ptr, dl.dtype, vocab, 0, x + r0 * hidden, BR_F32, hidden,
+        BR_OP(product(1, 0, vocab, hidden, rows, alpha, dl.ptr, dl.dtype, vocab, 0, x + r0 * hidden, BR_F32, hidden,
                       0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
     }
 

@@ -357,6 +357,13 @@ template <>
 __device__ __forceinline__ float cvt_out<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ __half cvt_out<__half>(float v) { return __float2half_rn(v); }
+template <>
+__device__ __forceinline__ void store4<__hip_bfloat16>(__hip_bfloat16* p, float a, float b, float c, float d) {
+    auto bits = [](float v) { return (unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(v)); };
+    *reinterpret_cast<uint2*>(p) = make_uint2(bits(a) | (bits(b) << 16), bits(c) | (bits(d) << 16));
+}
+template <>
+__device__ __forceinline__ __hip_bfloat16 cvt_out<__hip_bfloat16>(float v) { return __float2bfloat16(v); }
 
 template <typename OUT>
 __global__ __launch_bounds__(kVBlock) void nll_bwd_kernel(const float* logits, const int32_t* __restrict__ target,
@@ -507,6 +514,11 @@ int br_hip_logsoftmax_nll_bwd(const float* logits, const int32_t* target, const 
         const bool vec_ok = vocab % 4 == 0 && aligned16(logits) && aligned8(dlogits);
         nll_bwd_kernel<__half><<<(unsigned)rows, kVBlock, 0, st>>>(logits, target, keep, lse, (__half*)dlogits,
                                                                    scale, vocab, vec_ok);
+    } else if (dlogits_dtype == BR_BF16) {
+        if ((const void*)logits == dlogits) return BR_ERR_OUTPUT;
+        const bool vec_ok = vocab % 4 == 0 && aligned16(logits) && aligned8(dlogits);
+        nll_bwd_kernel<__hip_bfloat16><<<(unsigned)rows, kVBlock, 0, st>>>(logits, target, keep, lse,
+                                                                           (__hip_bfloat16*)dlogits, scale, vocab, vec_ok);
     } else {
         return BR_ERR_TODO;
     }

@@ -246,7 +246,11 @@ int br_hip_logsoftmax_nll_fwd(const float* logits, const int32_t* target, const 
 /* cudnnSoftmaxBackward(LOG) of cuda_tensor.cpp:656-668 applied to the seed
  * written by nll_loss.cu:33:
  *   dlogits[r,c] = keep[r] ? (exp(logits[r,c]-lse[r]) - [c==target[r]])*scale : 0
- * dlogits_dtype is BR_F32 or BR_F16; dlogits may alias logits when fp32. */
+ * dlogits_dtype is BR_F32, BR_F16 or BR_BF16; dlogits may alias logits when
+ * fp32.  A 16-bit dlogits that feeds matrix products should be written with a
+ * scale that keeps small probabilities representable (fp16 flushes below
+ * 3e-8): pass a power of two here and fold 1/count and its inverse into the
+ * products' alpha. */
 int br_hip_logsoftmax_nll_bwd(const float* logits, const int32_t* target, const int32_t* keep,
                               const float* lse, void* dlogits, int dlogits_dtype, float scale,
                               int64_t rows, int64_t vocab, br_stream_t stream);

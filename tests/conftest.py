@@ -27,15 +27,26 @@ def fixture_ids_mask():
 def assert_close(got, ref, rtol, what=""):
     """|got - ref| <= rtol * (|ref| + rms(ref)) elementwise: a relative bound
     with a floor tied to the tensor's own scale, so entries that are zero by
-    cancellation do not demand infinite precision."""
-    got = np.asarray(got, np.float64)
-    ref = np.asarray(ref, np.float64)
+    cancellation do not demand infinite precision.  Works through the arrays in
+    slices so that a gigabyte-sized gradient needs no fp64 copy of itself."""
+    got = np.asarray(got)
+    ref = np.asarray(ref)
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
-    assert np.all(np.isfinite(got)), what + ": non-finite values"
-    rms = float(np.sqrt(np.mean(ref * ref))) if ref.size else 0.0
-    bound = rtol * (np.abs(ref) + rms) + 1e-30
-    err = np.abs(got - ref)
-    worst = float(np.max(err / bound)) if ref.size else 0.0
+    got = got.reshape(-1)
+    ref = ref.reshape(-1)
+    step = 1 << 24
+    total = 0.0
+    for i in range(0, ref.size, step):
+        r = ref[i:i + step].astype(np.float64)
+        total += float(np.dot(r, r))
+    rms = float(np.sqrt(total / ref.size)) if ref.size else 0.0
+    worst = 0.0
+    for i in range(0, ref.size, step):
+        g = got[i:i + step].astype(np.float64)
+        r = ref[i:i + step].astype(np.float64)
+        assert np.all(np.isfinite(g)), what + ": non-finite values"
+        bound = rtol * (np.abs(r) + rms) + 1e-30
+        worst = max(worst, float(np.max(np.abs(g - r) / bound)))
     assert worst <= 1.0, "%s: worst error %.3g x the %.1e bound (rms %.3g)" % (
         what, worst, rtol, rms)
 

@@ -167,6 +167,44 @@ def test_loss_head_against_oracle(runtime, mode):
     env.close()
 
 
+def test_loss_head_at_the_true_vocabulary_keeps_small_probabilities(runtime):
+    """V = 250880, one 512-token sequence, fp16 products, a PEAKED head (logits
+    ~ N(0, 6)): most probabilities are far below 1e-5, and p / count would
+    fall under fp16's smallest subnormal.  The stored 16-bit gradient therefore
+    leaves 1/count to the products' alpha; checked on x_g, on the whole
+    lm_head_g, and row by row on vocabulary entries that are nobody's label and
+    whose largest probability lies in [1e-7, 1e-5] -- rows that a gradient
+    rounded to fp16 after the 1/count scaling would return as zeros."""
+    hidden, heads, batch, tokens, vocab = 1024, 8, 1, 512, 250880
+    env, _, x, _, mask, ids = setup_block(runtime, hidden, heads, batch, tokens, "f16", vocab=vocab)
+    rng = np.random.default_rng(15)
+    lm = (6.0 / np.sqrt(hidden) * rng.standard_normal((vocab, hidden))).astype(np.float16).astype(np.float32)
+    env.execute("%d %d 2 'cuda' 'f16' op.create 'lm_head.weight' !" % (vocab, hidden))
+    env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight_g' !  'lm_head.weight_g' @ op.zero" % (vocab, hidden))
+    env.write("lm_head.weight", lm)
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xa' @ 'lm_head.weight_g' @ "
+                "op.loss_backward op.sync")
+    loss_ref, xg_ref, wg_ref, _ = orc.loss_backward(x, ids, mask, lm)
+    labels, count = orc.loss_labels(ids, mask)
+    assert count == (tokens - tokens // 4) - 1
+    assert_close(env.read("xa"), xg_ref, 2e-2, "x_g at V=250880")
+    wg = env.read("lm_head.weight_g")
+    assert_close(wg, wg_ref, 2e-2, "lm_head_g at V=250880")
+    # selection only: probabilities from a plain numpy product
+    logits = x.reshape(tokens, hidden)[labels.reshape(-1) >= 0] @ lm.T
+    logits -= logits.max(axis=1, keepdims=True)
+    prob = np.exp(logits)
+    prob /= prob.sum(axis=1, keepdims=True)
+    largest = prob.max(axis=0)
+    rare = (largest >= 1e-7) & (largest <= 1e-5)
+    rare[labels[labels >= 0]] = False
+    assert rare.sum() > 1000
+    ref_rows = wg_ref[rare].astype(np.float64)
+    err = np.linalg.norm(wg[rare] - ref_rows, axis=1) / np.linalg.norm(ref_rows, axis=1)
+    assert float(err.max()) <= 2e-2, "rare-token rows of lm_head_g: worst relative row error %.3g" % float(err.max())
+    env.close()
+
+
 def test_loss_value_and_chunking(runtime, capfd):
     """The printed / returned value is +mean log-prob; a logits workspace that
     holds only a few rows forces the chunked path."""
@@ -466,3 +504,49 @@ def test_flash_attention_words_on_separate_and_packed_projections_agree(runtime)
             assert np.array_equal(packed[:, :, i * h:(i + 1) * h], env.read(n).reshape(b, t, h)), n
     finally:
         env.close()
+
+
+def test_block_at_the_full_headline_size_against_oracle(runtime):
+    """Config C4 exactly: hidden 4096, 32 heads x 128, FFN 16384, batch 4 x 512
+    tokens, fp16 weights (the last sequence right-padded).  The oracle's block
+    is computed once; the fp32-arena operator words (`block_step`) and the
+    fused-attention words the benchmark quotes (`block_step_flash`) are each
+    held to 2e-2 on the block output, the input gradient and every parameter
+    gradient.  This is the shape where the 256x256 GEMM tiles, split-K and the
+    8-key-tile attention loops run."""
+    hidden, heads, batch, tokens = 4096, 32, 4, 512
+    tol = 2e-2
+    print("case C4 full size", flush=True)
+    env, w, x, dy, mask, _ = setup_block(runtime, hidden, heads, batch, tokens, "f16")
+    saved = blk.layer_forward(w, x, orc.alibi(heads, tokens), orc.xmask(mask), heads, 1e-5)
+    dx_ref, g_ref = blk.layer_backward(w, saved, x, dy, heads, 1e-5)
+    out_ref = saved["xa"]
+    qkv_w = np.concatenate([g_ref["query.weight_g"], g_ref["key.weight_g"], g_ref["value.weight_g"]])
+    qkv_b = np.concatenate([g_ref["query.bias_g"], g_ref["key.bias_g"], g_ref["value.bias_g"]])
+    v_only = slice(2 * hidden, 3 * hidden)
+    del saved
+
+    def check(step_word, forward_word, what):
+        print("  path", what, flush=True)
+        env.write("xinput", x)
+        env.write("yout_g", dy)
+        env.execute("zero_layer_grad")
+        env.execute(step_word + " op.sync")
+        assert_close(env.read("xa"), dx_ref, tol, what + ": dx")
+        for name, ref in g_ref.items():
+            if name.startswith(("query.", "key.", "value.")):
+                continue
+            assert_close(env.read(name).reshape(ref.shape), ref, tol, what + ": " + name)
+        assert_close(env.read("query_key_value.weight_g"), qkv_w, tol, what + ": query_key_value.weight_g")
+        # the key third of the bias gradient is zero up to rounding; query and value thirds are checked
+        got_b = env.read("query_key_value.bias_g")
+        assert_close(got_b[:hidden], qkv_b[:hidden], tol, what + ": query bias_g")
+        assert_close(got_b[v_only], qkv_b[v_only], tol, what + ": value bias_g")
+        env.write("xinput", x)
+        env.execute(forward_word + " op.sync")
+        assert_close(env.read("xa"), out_ref, tol, what + ": block output")
+
+    check("block_step", "layer_forward", "operator words")
+    env.execute("create_operand_buffers create_flash_buffers prepare_batch_flash")
+    check("block_step_flash", "layer_forward_flash", "fused-attention words")
+    env.close()

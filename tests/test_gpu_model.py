@@ -52,6 +52,10 @@ def build(mode, layers, batch, tokens, hidden, heads, vocab, seed):
     ("f16", 2, 2, 64, 512, 8, 2048),
     ("f16", 2, 2, 64, 512, 4, 2048),      # head size 128: attention runs as the fused kernels
     ("bf16", 2, 2, 64, 512, 4, 2048),     # the same in bf16 (8-bit mantissa; see the bound below)
+    # config C5's shapes with two of its thirty blocks: one 512-token sequence, hidden 4096, 32 heads,
+    # the 250880-word tied table (products with M = 512: few output tiles, split along K; one logits
+    # row per position)
+    ("f16", 2, 1, 512, 4096, 32, 250880),
 ])
 def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden, heads, vocab):
     print("case %s layers=%d batch=%d tokens=%d hidden=%d" % (mode, layers, batch, tokens, hidden), flush=True)
