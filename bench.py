@@ -263,7 +263,7 @@ def elementwise_leg(hip, timer, torch):
     rec("layernorm_fwd [2048,4096] f32", sec, 2 * rows * cols * 4)
     ws = torch.empty(lib.br_hip_layernorm_bwd_workspace(rows, cols), dtype=torch.uint8, device="cuda")
     sec = timer.run(lambda i: hip.call("br_hip_layernorm_bwd", vp(dys[i % nb]), vp(ys[i % nb]), vp(g), vp(b), vp(var),
-                                       vp(dg), vp(db), vp(dxs[i % nb]), rows, cols, 1e-5, vp(ws), ws.numel(), st),
+                                       vp(dg), vp(db), vp(dxs[i % nb]), rows, cols, 1e-5, 1.0, vp(ws), ws.numel(), st),
                     200, 10)
     rec("layernorm_bwd [2048,4096] f32", sec, 3 * rows * cols * 4)
     del xs, ys, dys, dxs

@@ -63,6 +63,7 @@ struct Embed : public NativeWord {
 };
 
 // ( ids dx grad -- )  grad[ids[i], :] += dx[i, :]: the gather's backward
+// (dx carries the gradient lift of the backward pass, the table's gradient does not)
 struct EmbedBackward : public NativeWord {
     void run(Stack& stack) override {
         tensor_t grad = stack.pop_tensor();
@@ -81,7 +82,7 @@ struct EmbedBackward : public NativeWord {
         BR_HIP_CHECK(br_hip_memcpy_h2d(d_ids, ids->data(), (size_t)n * sizeof(int32_t), ComputingContext::stream));
         BR_HIP_CHECK(br_hip_embedding_scatter_add(static_cast<const float*>(dx->data()), d_ids,
                                                   static_cast<float*>(grad->data()), n, hidden, vocab,
-                                                  ComputingContext::stream));
+                                                  1.0f / ComputingContext::grad_lift, ComputingContext::stream));
     }
     NWORD_CREATOR_DEFINE_LR(EmbedBackward)
 };
@@ -162,11 +163,18 @@ struct LastLoss : public NativeWord {
     NWORD_CREATOR_DEFINE_LR(LastLoss)
 };
 
+// ( -- S )  the gradient lift the current backward pass carries (1 = none)
+struct GradLiftValue : public NativeWord {
+    void run(Stack& stack) override { stack.push_number((double)ComputingContext::grad_lift); }
+    NWORD_CREATOR_DEFINE_LR(GradLiftValue)
+};
+
 }  // namespace
 
 void load_bloom_words(Enviroment& env) {
     env.insert_native_word("bloom.normal", Normal::creator);
     env.insert_native_word("bloom.last_loss", LastLoss::creator);
+    env.insert_native_word("bloom.grad_lift", GradLiftValue::creator);
     env.insert_native_word("bloom.embed", Embed::creator);
     env.insert_native_word("bloom.embed_backward", EmbedBackward::creator);
     env.insert_native_word("bloom.alibi", Alibi::creator);

@@ -154,7 +154,14 @@ float BloomTrainer::step(const int32_t* ids, const int32_t* mask) {
     tensor_t t_mask = env_.hash().find_tensor("mask_");
     memcpy(t_ids->data(), ids, n * sizeof(int32_t));
     memcpy(t_mask->data(), mask, n * sizeof(int32_t));
+    // 16-bit products: the loss head picks a gradient lift for this step's
+    // backward pass; the setting is this step's only (the context is global)
+    ComputingContext::grad_lift_auto = cfg_.gemm_precision != "f32" && cfg_.gemm_precision != "float";
+    ComputingContext::grad_lift = 1.0f;
     env_.run(step_.get());
+    grad_lift_ = ComputingContext::grad_lift;
+    ComputingContext::grad_lift_auto = false;
+    ComputingContext::grad_lift = 1.0f;
     return ComputingContext::last_loss;
 }
 

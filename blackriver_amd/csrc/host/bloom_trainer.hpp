@@ -41,6 +41,11 @@ public:
     // One step: ids / mask are [batch, tokens] int32 on the host.  Returns the
     // mean log-probability of the labels (the sign convention of op.loss_backward).
     float step(const int32_t* ids, const int32_t* mask);
+    // The power of two the last step's backward pass carried on its activation
+    // gradients (what is left in the blocks' and hash 0's gradient buffers, e.g.
+    // the embedding rows' gradient `xc`, is that many times the true gradient;
+    // parameter gradients are at their true scale).  1 with fp32 products.
+    float grad_lift() const { return grad_lift_; }
 
     // AdamW state for every parameter (moments; fp32 master copies of 16-bit
     // matrices, initialised from the matrices as they are now: call after the
@@ -67,6 +72,7 @@ private:
     bool masters() const { return cfg_.weight_dtype != "float"; }
     bool has_optimizer_ = false;
     int64_t adam_step_ = 0;
+    float grad_lift_ = 1.0f;
 };
 
 }  // namespace br

@@ -305,6 +305,14 @@ int br_bloom_model_step(br_env_t* e, const int32_t* ids, const int32_t* mask, fl
     });
 }
 
+int br_bloom_model_grad_lift(br_env_t* e, float* lift) {
+    return guarded([&]() {
+        br_assert(e->trainer != nullptr, "br_bloom_model_create has not run");
+        br_assert(lift != nullptr, "br_bloom_model_grad_lift: null output");
+        *lift = e->trainer->grad_lift();
+    });
+}
+
 int br_bloom_model_optimizer_create(br_env_t* e, float lr, float beta1, float beta2, float eps, float weight_decay) {
     return guarded([&]() {
         br_assert(e->trainer != nullptr, "br_bloom_model_create has not run");

@@ -84,6 +84,9 @@ struct Operand {
     const void* ptr;
     int dtype;
 };
+// Factor that takes the backward pass's gradient lift out of a parameter gradient.
+float unlift() { return 1.0f / ComputingContext::grad_lift; }
+
 Operand shared_operand(const void* p, int dtype, int64_t items, int compute) {
     if (dtype != BR_F32 || compute == BR_GEMM_F32 || items % 8 != 0) return {p, dtype};
     const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
@@ -97,7 +100,7 @@ Operand shared_operand(const void* p, int dtype, int64_t items, int compute) {
 // x_g[n,in] = dy . W (in that order: x_g may overwrite x).
 int linear_backward_products(const Operand& dy, const tensor_t& x, const tensor_t& weight, const tensor_t& x_g,
                              const tensor_t& weight_g, int64_t n, int64_t in, int64_t out, int compute) {
-    int rc = product(1, 0, out, in, n, 1.0f, dy.ptr, dy.dtype, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
+    int rc = product(1, 0, out, in, n, unlift(), dy.ptr, dy.dtype, out, 0, x->data(), code(x), in, 0, 0, weight_g->data(),
                      code(weight_g), in, 0, nullptr, 1, compute);
     if (rc != BR_OK) return rc;
     return product(0, 0, n, in, out, 1.0f, dy.ptr, dy.dtype, out, 0, weight->data(), code(weight), in, 0, 0,
@@ -439,6 +442,18 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
         }
     }
     const float scale = count > 0 ? 1.0f / (float)count : 0.0f;
+    const int compute = pick_compute({self, lm_head});
+    if (ComputingContext::grad_lift_auto) {
+        // 16 * 2^ceil(log2(count)): undoes the mean over loss positions and leaves
+        // four more bits of headroom below; no lift for fp32 products
+        float lift_now = 1.0f;
+        if (compute != BR_GEMM_F32 && count > 0) {
+            lift_now = 16.0f;
+            while (lift_now < 16.0f * (float)count) lift_now *= 2.0f;
+        }
+        ComputingContext::grad_lift = lift_now;
+    }
+    const float grad_lift = ComputingContext::grad_lift;   // x_g leaves carrying this factor
 
     // small per-row arrays in the workspace tail (slots 2..7)
     br_assert((size_t)n * 4 * sizeof(float) + 64 <= 6u * (1u << 20), "too many rows for the loss scratch");
@@ -465,7 +480,6 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
     }
 
     BR_OP(br_hip_fill(x_g->data(), BR_F32, 0.f, n * hidden, stream()));
-    const int compute = pick_compute({self, lm_head});
     const float* x = static_cast<const float*>(mem_);
     float* dx = static_cast<float*>(x_g->data());
     float* logits = static_cast<float*>(all_logits->data());
@@ -504,7 +518,7 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
                 dl = shared_operand(logits, BR_F32, rows * vocab, compute);
             }
         }
-        BR_OP(product(0, 0, rows, hidden, vocab, alpha, dl.ptr, dl.dtype, vocab, 0, lm_head->data(), code(lm_head),
+        BR_OP(product(0, 0, rows, hidden, vocab, alpha * grad_lift, dl.ptr, dl.dtype, vocab, 0, lm_head->data(), code(lm_head),
                       hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute));
         BR_OP(product(1, 0, vocab, hidden, rows, alpha, dl.ptr, dl.dtype, vocab, 0, x + r0 * hidden, BR_F32, hidden,
                       0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
@@ -556,7 +570,7 @@ ComputingReturn HIPTensor<DT>::op_layernorm_backward(tensor_t self, tensor_t sca
                                static_cast<const float*>(scale->data()), static_cast<const float*>(bias->data()),
                                static_cast<const float*>(var->data()), static_cast<float*>(dscale->data()),
                                static_cast<float*>(dbias->data()), static_cast<float*>(din->data()), rows, cols, eps,
-                               ws, need, stream()));
+                               unlift(), ws, need, stream()));
     return OP_OK;
 }
 
@@ -583,10 +597,10 @@ ComputingReturn HIPTensor<DT>::op_linear_backward(tensor_t self, tensor_t x, ten
         const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
         void* dy16 = ComputingContext::gemm_staging(1, (size_t)(n * out) * 2);
         BR_OP(br_hip_colsum_cast(static_cast<const float*>(mem_), static_cast<float*>(bias_g->data()), dy16, native, n,
-                                 out, ws, need, stream()));
+                                 out, unlift(), ws, need, stream()));
         dy = Operand{dy16, native};
     } else {
-        BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, ws, need, stream()));
+        BR_OP(br_hip_colsum(mem_, (int)DT, static_cast<float*>(bias_g->data()), n, out, unlift(), ws, need, stream()));
         dy = shared_operand(mem_, (int)DT, n * out, compute);
     }
     BR_OP(linear_backward_products(dy, x, weight, x_g, weight_g, n, in, out, compute));
@@ -719,8 +733,8 @@ ComputingReturn hip_gelu_linear_backward(const tensor_t& dy, const tensor_t& u, 
             void* dy16 = ComputingContext::gemm_staging(1, (size_t)(n * out) * 2);
             const int rc = br_hip_gelu_bwd_colsum_cast(
                 static_cast<const float*>(dy->data()), static_cast<const float*>(u->data()),
-                static_cast<float*>(du->data()), static_cast<float*>(bias_g->data()), dy16, native, n, out, ws, need,
-                stream());
+                static_cast<float*>(du->data()), static_cast<float*>(bias_g->data()), dy16, native, n, out, unlift(), ws,
+                need, stream());
             if (rc != BR_ERR_TODO) {
                 BR_OP(rc);
                 BR_OP(linear_backward_products(Operand{dy16, native}, x, weight, x_g, weight_g, n, in, out, compute));
@@ -766,7 +780,7 @@ ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& s
                 static_cast<const float*>(scale->data()), static_cast<const float*>(bias->data()),
                 static_cast<const float*>(var->data()), static_cast<const float*>(residual->data()),
                 static_cast<float*>(dscale->data()), static_cast<float*>(dbias->data()),
-                static_cast<float*>(din->data()), rows, cols, eps, ws, need, stream());
+                static_cast<float*>(din->data()), rows, cols, eps, unlift(), ws, need, stream());
             if (rc != BR_ERR_TODO) return done(rc, "br_hip_layernorm_bwd_residual");
         }
     }

@@ -54,6 +54,8 @@ size_t ComputingContext::workspace_size = 0;
 int ComputingContext::fp32_gemm_compute = BR_GEMM_F32;
 float ComputingContext::last_loss = 0.0f;
 bool ComputingContext::echo_loss = true;
+float ComputingContext::grad_lift = 1.0f;
+bool ComputingContext::grad_lift_auto = false;
 void* ComputingContext::scratch_ptr_ = nullptr;
 size_t ComputingContext::scratch_size_ = 0;
 void* ComputingContext::staging_ptr_[2] = {nullptr, nullptr};

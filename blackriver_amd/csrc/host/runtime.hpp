@@ -31,6 +31,16 @@ struct ComputingContext {
     // op_loss_backward prints "#################  <count> <loss>" like the
     // reference (cuda_tensor.cpp:692) unless a driver turns it off
     static bool echo_loss;
+    // Gradient lift S (a power of two, 1 = off): op_loss_backward hands out
+    // x_g = S * dL/dx, every backward operator passes the factor on through its
+    // activation gradient and takes it out of the parameter gradients it writes
+    // (1/S in the weight-gradient product's alpha and in the bias / LayerNorm
+    // sums), so parameter gradients always come out at their true scale.  With
+    // 16-bit products this keeps the small gradients of a mean-over-tokens loss
+    // clear of fp16's subnormal range.  grad_lift_auto: op_loss_backward picks
+    // S = 16 * 2^ceil(log2(count)) itself when the products run in 16 bit.
+    static float grad_lift;
+    static bool grad_lift_auto;
 
     static void boot(int dev);  // 128 MiB of scratch like context.cpp:31
     static void shutdown();

@@ -4,6 +4,8 @@
 // (blackriver/nn.cpp:16-337) so the model scripts run unchanged.
 #include "words.hpp"
 
+#include <cmath>
+
 #include <vector>
 
 #include "br_hip.h"
@@ -77,6 +79,23 @@ BR_WORD(GemmPrecision,
     else if (p == "f16") ComputingContext::fp32_gemm_compute = BR_GEMM_F16;
     else if (p == "bf16") ComputingContext::fp32_gemm_compute = BR_GEMM_BF16;
     else br_panic("op.gemm_precision takes \"f32\", \"f16\" or \"bf16\"");
+)
+
+// ( S -- )  gradient lift for the backward pass (extension): S > 0 must be a
+// power of two and is used as given; 0 lets op.loss_backward choose it from the
+// number of loss positions; 1 (the default) switches it off.
+BR_WORD(GradLift,
+    const double v = stack.pop_number();
+    if (v == 0.0) {
+        ComputingContext::grad_lift_auto = true;
+        ComputingContext::grad_lift = 1.0f;
+    } else {
+        int e = 0;
+        br_assert(v > 0.0 && std::frexp(v, &e) == 0.5 && v <= 16777216.0 && v >= 1.0 / 16777216.0,
+                  "op.grad_lift takes 0 (choose per step) or a power of two");
+        ComputingContext::grad_lift_auto = false;
+        ComputingContext::grad_lift = (float)v;
+    }
 )
 
 BR_WORD(Zero, tensor_t t = stack.pop_tensor(); t->op_zero(t);)
@@ -423,6 +442,7 @@ void load_nn_words(Enviroment& env) {
         {"op.sync", Sync::creator},
         {"op.create", Create::creator},
         {"op.gemm_precision", GemmPrecision::creator},
+        {"op.grad_lift", GradLift::creator},
         {"op.zero", Zero::creator},
         {"op.fill", Fill::creator},
         {"op.view", View::creator},

@@ -430,12 +430,12 @@ __global__ __launch_bounds__(kBlock) void colsum_partial(const T* x, float* part
 
 // Stage 2: out[c] = sum_g partial[g][c]  (fixed order: deterministic).
 __global__ __launch_bounds__(kBlock) void colsum_final(const float* partial, float* out, int groups,
-                                                        int64_t cols) {
+                                                        int64_t cols, float scale) {
     const int64_t col = (int64_t)blockIdx.x * kBlock + threadIdx.x;
     if (col >= cols) return;
     float acc = 0.f;
     for (int g = 0; g < groups; g++) acc += partial[(int64_t)g * cols + col];
-    out[col] = acc;
+    out[col] = acc * scale;
 }
 
 // Vector forms of the two stages (cols % VEC == 0, 16-byte aligned rows).
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(kBlock) void gelu_bwd_colsum_cast_partial(const flo
 // groups, every load of a workgroup in flight at once; slices are combined in
 // LDS in a fixed order.
 __global__ __launch_bounds__(1024) void colsum_final_x4(const float4* __restrict__ partial, float4* __restrict__ out,
-                                                        int groups, int cols4) {
+                                                        int groups, int cols4, float scale) {
     __shared__ float4 l[64][16];
     const int q = threadIdx.x & 15, sl = threadIdx.x >> 4;
     const int c4 = blockIdx.x * 16 + q;
@@ -595,18 +595,18 @@ __global__ __launch_bounds__(1024) void colsum_final_x4(const float4* __restrict
             const float4 a = l[k][q];
             s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
         }
-        out[c4] = s;
+        out[c4] = make_float4(s.x * scale, s.y * scale, s.z * scale, s.w * scale);
     }
 }
 
 // Launches stage 2 in its vector form when the shapes allow.
-int colsum_finish(const float* partial, float* out, int groups, int64_t cols, hipStream_t st) {
+int colsum_finish(const float* partial, float* out, int groups, int64_t cols, float scale, hipStream_t st) {
     if (cols % 4 == 0 && aligned16(partial) && aligned16(out))
         colsum_final_x4<<<(unsigned)((cols / 4 + 15) / 16), 1024, 0, st>>>(reinterpret_cast<const float4*>(partial),
                                                                             reinterpret_cast<float4*>(out), groups,
-                                                                            (int)(cols / 4));
+                                                                            (int)(cols / 4), scale);
     else
-        colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>(partial, out, groups, cols);
+        colsum_final<<<(unsigned)((cols + kBlock - 1) / kBlock), kBlock, 0, st>>>(partial, out, groups, cols, scale);
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }
@@ -758,7 +758,7 @@ __global__ __launch_bounds__(kBlock) void normal_kernel(T* dst, float mean, floa
 // row, in ascending position order, starting from the row's current value.
 __global__ __launch_bounds__(kBlock) void scatter_add_rows(const float* __restrict__ dx,
                                                             const int32_t* __restrict__ ids, float* grad, int n,
-                                                            int64_t hidden, int64_t vocab, bool vec) {
+                                                            int64_t hidden, int64_t vocab, float scale, bool vec) {
     const int i = blockIdx.x;
     const int32_t id = ids[i];
     if (id < 0 || (int64_t)id >= vocab) return;
@@ -773,7 +773,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_rows(const float* __restri
             for (int j = i; j < n; j++) {
                 if (ids[j] != id) continue;
                 const float4 d = reinterpret_cast<const float4*>(dx + (int64_t)j * hidden)[c];
-                acc.x += d.x; acc.y += d.y; acc.z += d.z; acc.w += d.w;
+                acc.x += d.x * scale; acc.y += d.y * scale; acc.z += d.z * scale; acc.w += d.w * scale;
             }
             reinterpret_cast<float4*>(row)[c] = acc;
         }
@@ -781,7 +781,7 @@ __global__ __launch_bounds__(kBlock) void scatter_add_rows(const float* __restri
         for (int64_t c = threadIdx.x; c < hidden; c += kBlock) {
             float acc = row[c];
             for (int j = i; j < n; j++)
-                if (ids[j] == id) acc += dx[(int64_t)j * hidden + c];
+                if (ids[j] == id) acc += dx[(int64_t)j * hidden + c] * scale;
             row[c] = acc;
         }
     }
@@ -1037,11 +1037,11 @@ int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void*
             gelu_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>((const __half*)dy, (const __half*)x,
                                                                        bias, (__half*)dx, n, cols, true);
         BR_HIP_LAUNCH_CHECK();
-        if (dbias) return br_hip_colsum(dx, dtype, dbias, rows, cols, workspace, workspace_bytes, stream);
+        if (dbias) return br_hip_colsum(dx, dtype, dbias, rows, cols, 1.0f, workspace, workspace_bytes, stream);
         return BR_OK;
     }
     BR_HIP_LAUNCH_CHECK();
-    if (dbias) return colsum_finish(partial, dbias, groups, cols, st);
+    if (dbias) return colsum_finish(partial, dbias, groups, cols, 1.0f, st);
     return BR_OK;
 }
 
@@ -1053,7 +1053,7 @@ size_t br_hip_colsum_workspace(int64_t rows, int64_t cols) {
     return strips > vec ? strips : vec;
 }
 
-int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols, void* workspace,
+int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols, float out_scale, void* workspace,
                   size_t workspace_bytes, br_stream_t stream) {
     if (rows < 0 || cols <= 0) return BR_ERR_ATTR;
     if (!out) return BR_ERR_OUTPUT;
@@ -1074,7 +1074,7 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
         else
             colsum_partial_vec<__half, 8><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
         BR_HIP_LAUNCH_CHECK();
-        return colsum_finish(partial, out, groups, cols, st);
+        return colsum_finish(partial, out, groups, cols, out_scale, st);
     }
     const int rpb = strip_rows(rows);
     const int groups = (int)((rows + rpb - 1) / rpb);
@@ -1084,11 +1084,11 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
     else
         colsum_partial<__half><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
-    return colsum_finish(partial, out, groups, cols, st);
+    return colsum_finish(partial, out, groups, cols, out_scale, st);
 }
 
 int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int64_t rows, int64_t cols,
-                       void* workspace, size_t workspace_bytes, br_stream_t stream) {
+                       float out_scale, void* workspace, size_t workspace_bytes, br_stream_t stream) {
     if (rows <= 0 || cols <= 0) return BR_ERR_ATTR;
     if (!x) return BR_ERR_INPUT;
     if (!out || !x16) return BR_ERR_OUTPUT;
@@ -1106,11 +1106,11 @@ int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int
     else
         colsum_cast_partial<__hip_bfloat16><<<grid, kBlock, 0, st>>>(x, partial, (__hip_bfloat16*)x16, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
-    return colsum_finish(partial, out, groups, cols, st);
+    return colsum_finish(partial, out, groups, cols, out_scale, st);
 }
 
 int br_hip_gelu_bwd_colsum_cast(const float* dy, const float* x, float* dx, float* out, void* dx16, int dx16_dtype,
-                                int64_t rows, int64_t cols, void* workspace, size_t workspace_bytes,
+                                int64_t rows, int64_t cols, float out_scale, void* workspace, size_t workspace_bytes,
                                 br_stream_t stream) {
     if (rows <= 0 || cols <= 0) return BR_ERR_ATTR;
     if (!dy || !x) return BR_ERR_INPUT;
@@ -1133,7 +1133,7 @@ int br_hip_gelu_bwd_colsum_cast(const float* dy, const float* x, float* dx, floa
         gelu_bwd_colsum_cast_partial<__hip_bfloat16><<<grid, kBlock, 0, st>>>(dy, x, dx, partial,
                                                                              (__hip_bfloat16*)dx16, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
-    return colsum_finish(partial, out, groups, cols, st);
+    return colsum_finish(partial, out, groups, cols, out_scale, st);
 }
 
 int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, int64_t s1, int64_t s2,
@@ -1183,13 +1183,13 @@ int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, in
 }
 
 int br_hip_embedding_scatter_add(const float* dx, const int32_t* ids, float* grad, int64_t n, int64_t hidden,
-                                 int64_t vocab, br_stream_t stream) {
+                                 int64_t vocab, float dx_scale, br_stream_t stream) {
     if (n < 0 || hidden <= 0 || vocab <= 0 || n > 0x7fffffff) return BR_ERR_ATTR;
     if (n == 0) return BR_OK;
     if (!dx || !ids) return BR_ERR_INPUT;
     if (!grad || (const float*)grad == dx) return BR_ERR_OUTPUT;
     const bool vec = hidden % 4 == 0 && aligned16(dx) && aligned16(grad);
-    scatter_add_rows<<<(unsigned)n, kBlock, 0, as_stream(stream)>>>(dx, ids, grad, (int)n, hidden, vocab, vec);
+    scatter_add_rows<<<(unsigned)n, kBlock, 0, as_stream(stream)>>>(dx, ids, grad, (int)n, hidden, vocab, dx_scale, vec);
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }

@@ -262,7 +262,8 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_cols_generic(const float* dy, c
 // dgamma[c] = sum_p part_dgamma[p][c] (and dbeta likewise), fixed order.
 // blockDim = (64 columns, 4 slices of partials); slices are combined in LDS.
 __global__ __launch_bounds__(kBlock) void ln_bwd_finalize(const float* part_dgamma, const float* part_dbeta,
-                                                           float* dgamma, float* dbeta, int parts, int64_t cols) {
+                                                           float* dgamma, float* dbeta, int parts, int64_t cols,
+                                                           float scale) {
     __shared__ float lg[4][64], lb[4][64];
     const int cx = threadIdx.x & 63, sl = threadIdx.x >> 6;
     const int64_t c = (int64_t)blockIdx.x * 64 + cx;
@@ -277,8 +278,8 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_finalize(const float* part_dgam
     lb[sl][cx] = sb;
     __syncthreads();
     if (sl == 0 && c < cols) {
-        dgamma[c] = (lg[0][cx] + lg[1][cx]) + (lg[2][cx] + lg[3][cx]);
-        dbeta[c] = (lb[0][cx] + lb[1][cx]) + (lb[2][cx] + lb[3][cx]);
+        dgamma[c] = ((lg[0][cx] + lg[1][cx]) + (lg[2][cx] + lg[3][cx])) * scale;
+        dbeta[c] = ((lb[0][cx] + lb[1][cx]) + (lb[2][cx] + lb[3][cx])) * scale;
     }
 }
 
@@ -290,7 +291,7 @@ constexpr int kFinSlices = 64;
 __global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restrict__ part_dgamma,
                                                            const float4* __restrict__ part_dbeta,
                                                            float4* __restrict__ dgamma, float4* __restrict__ dbeta,
-                                                           int parts, int cols4) {
+                                                           int parts, int cols4, float scale) {
     __shared__ float4 lg[kFinSlices][16], lb[kFinSlices][16];
     const int q = threadIdx.x & 15, sl = threadIdx.x >> 4;
     const int c4 = blockIdx.x * 16 + q;
@@ -322,8 +323,8 @@ __global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restr
             sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
             sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
         }
-        dgamma[c4] = sg;
-        dbeta[c4] = sb;
+        dgamma[c4] = make_float4(sg.x * scale, sg.y * scale, sg.z * scale, sg.w * scale);
+        dbeta[c4] = make_float4(sb.x * scale, sb.y * scale, sb.z * scale, sb.w * scale);
     }
 }
 
@@ -406,8 +407,8 @@ size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols) {
 
 static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamma, const float* beta,
                               const float* var, const float* residual, float* dgamma, float* dbeta, float* dx,
-                              int64_t rows, int64_t cols, float eps, void* workspace, size_t workspace_bytes,
-                              br_stream_t stream) {
+                              int64_t rows, int64_t cols, float eps, float param_scale, void* workspace,
+                              size_t workspace_bytes, br_stream_t stream) {
     if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
     if (!dgamma || !dbeta) return BR_ERR_OUTPUT;
     if (rows == 0) {
@@ -445,9 +446,9 @@ static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamm
         if (aligned16(dgamma) && aligned16(dbeta))
             ln_bwd_finalize_x4<<<(unsigned)((cols4 + 15) / 16), 1024, 0, st>>>(
                 reinterpret_cast<const float4*>(part_g), reinterpret_cast<const float4*>(part_b),
-                reinterpret_cast<float4*>(dgamma), reinterpret_cast<float4*>(dbeta), parts, cols4);
+                reinterpret_cast<float4*>(dgamma), reinterpret_cast<float4*>(dbeta), parts, cols4, param_scale);
         else
-            ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols);
+            ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols, param_scale);
     } else {
         const int rpb = strip_rows(rows);
         parts = (int)((rows + rpb - 1) / rpb);
@@ -458,7 +459,7 @@ static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamm
         BR_HIP_LAUNCH_CHECK();
         ln_bwd_dx_generic<<<(unsigned)rows, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, cols, eps);
         BR_HIP_LAUNCH_CHECK();
-        ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols);
+        ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols, param_scale);
     }
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
@@ -466,19 +467,19 @@ static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamm
 
 int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, const float* beta,
                          const float* var, float* dgamma, float* dbeta, float* dx, int64_t rows, int64_t cols,
-                         float eps, void* workspace, size_t workspace_bytes, br_stream_t stream) {
-    return layernorm_bwd_impl(dy, y, gamma, beta, var, nullptr, dgamma, dbeta, dx, rows, cols, eps, workspace,
-                              workspace_bytes, stream);
+                         float eps, float param_scale, void* workspace, size_t workspace_bytes, br_stream_t stream) {
+    return layernorm_bwd_impl(dy, y, gamma, beta, var, nullptr, dgamma, dbeta, dx, rows, cols, eps, param_scale,
+                              workspace, workspace_bytes, stream);
 }
 
 int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* gamma, const float* beta,
                                   const float* var, const float* residual, float* dgamma, float* dbeta, float* dx,
-                                  int64_t rows, int64_t cols, float eps, void* workspace, size_t workspace_bytes,
-                                  br_stream_t stream) {
+                                  int64_t rows, int64_t cols, float eps, float param_scale, void* workspace,
+                                  size_t workspace_bytes, br_stream_t stream) {
     if (rows > 0 && !residual) return BR_ERR_INPUT;
     if (rows == 0) residual = nullptr;
-    return layernorm_bwd_impl(dy, y, gamma, beta, var, residual, dgamma, dbeta, dx, rows, cols, eps, workspace,
-                              workspace_bytes, stream);
+    return layernorm_bwd_impl(dy, y, gamma, beta, var, residual, dgamma, dbeta, dx, rows, cols, eps, param_scale,
+                              workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -55,14 +55,14 @@ SIGNATURES = {
     "br_hip_bias_gelu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _vp, _sz, _vp]),
     "br_hip_transpose_0213": (_int, [_vp, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "br_hip_colsum_workspace": (_sz, [_i64, _i64]),
-    "br_hip_colsum_cast": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp, _sz, _vp]),
-    "br_hip_colsum": (_int, [_vp, _int, _vp, _i64, _i64, _vp, _sz, _vp]),
-    "br_hip_gelu_bwd_colsum_cast": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _vp, _sz, _vp]),
+    "br_hip_colsum_cast": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _vp, _sz, _vp]),
+    "br_hip_colsum": (_int, [_vp, _int, _vp, _i64, _i64, _f32, _vp, _sz, _vp]),
+    "br_hip_gelu_bwd_colsum_cast": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _f32, _vp, _sz, _vp]),
     "br_hip_layernorm_fwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp]),
     "br_hip_layernorm_fwd_copy16": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _f32, _vp]),
     "br_hip_layernorm_bwd_workspace": (_sz, [_i64, _i64]),
-    "br_hip_layernorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _vp, _sz, _vp]),
-    "br_hip_layernorm_bwd_residual": (_int, [_vp] * 9 + [_i64, _i64, _f32, _vp, _sz, _vp]),
+    "br_hip_layernorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _f32, _vp, _sz, _vp]),
+    "br_hip_layernorm_bwd_residual": (_int, [_vp] * 9 + [_i64, _i64, _f32, _f32, _vp, _sz, _vp]),
     "br_hip_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "br_hip_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "br_hip_softmax_bwd_to16": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp]),
@@ -81,7 +81,7 @@ SIGNATURES = {
     "br_hip_flash_attn_bwd": (_int, [_vp] * 5 + [_int] + [_vp] * 7 + [_i64] * 9 + [_vp]),
     "br_hip_adamw": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _i64, _f32, _f32, _f32, _f32, _f32, _i64, _vp]),
     "br_hip_embedding_gather": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
-    "br_hip_embedding_scatter_add": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp]),
+    "br_hip_embedding_scatter_add": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),
     "br_hip_alibi_table": (_int, [_vp, _i64, _i64, _vp]),
     "br_hip_xmask_table": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "br_hip_alibi_slopes": (_int, [ctypes.POINTER(ctypes.c_double), _i64]),

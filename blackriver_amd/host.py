@@ -56,6 +56,7 @@ SIGNATURES = {
     "br_bloom_model_set_fused_attention": (_int, [_vp, _int]),
     "br_bloom_model_init": (_int, [_vp, ctypes.c_uint64, ctypes.c_float]),
     "br_bloom_model_step": (_int, [_vp, _i32p, _i32p, ctypes.POINTER(ctypes.c_float)]),
+    "br_bloom_model_grad_lift": (_int, [_vp, ctypes.POINTER(ctypes.c_float)]),
     "br_bloom_model_optimizer_create": (_int, [_vp] + [ctypes.c_float] * 5),
     "br_bloom_model_optimizer_step": (_int, [_vp]),
     "br_bloom_fetch_data": (_int, [_i32p, _i32p, _i64, _i64, _f32p, _i64, _i64, _f32p, _f32p, _f32p]),
@@ -268,6 +269,13 @@ class BloomModel:
         _check(load().br_bloom_model_step(self.env._h, ids.ctypes.data_as(_i32p), mask.ctypes.data_as(_i32p),
                                           ctypes.byref(loss)), "model_step")
         return loss.value
+
+    def grad_lift(self) -> float:
+        """Power of two the last step's activation gradients were carried at
+        (parameter gradients are at their true scale)."""
+        v = ctypes.c_float()
+        _check(load().br_bloom_model_grad_lift(self.env._h, ctypes.byref(v)), "grad_lift")
+        return v.value
 
     def create_optimizer(self, lr=1e-4, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.0):
         """AdamW state (moments, fp32 masters of 16-bit matrices).  Call after

@@ -124,9 +124,12 @@ int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, in
                           int64_t s2, int64_t s3, br_stream_t stream);
 
 /* cudnnReduceTensor(ADD) of cuda_tensor.cpp:738-760: out[c] = sum_r x[r,c]
- * (x fp32 or fp16, out fp32).  workspace: br_hip_colsum_workspace bytes. */
+ * (x fp32 or fp16, out fp32), times out_scale (1 for the plain sum; a
+ * backward pass that carries its activation gradients lifted by a power of two
+ * S passes 1/S here to get the bias gradient at its true scale).
+ * workspace: br_hip_colsum_workspace bytes. */
 size_t br_hip_colsum_workspace(int64_t rows, int64_t cols);
-int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols,
+int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t cols, float out_scale,
                   void* workspace, size_t workspace_bytes, br_stream_t stream);
 /* The same column sums of an fp32 x together with a 16-bit copy of x (x16,
  * BR_F16 or BR_BF16, dense [rows, cols]) in one pass: op_linear_backward
@@ -134,7 +137,7 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
  * 16-bit MFMA type, the copy as the operand of its two products.  cols % 4 == 0,
  * x 16-byte aligned; workspace as for br_hip_colsum. */
 int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int64_t rows, int64_t cols,
-                       void* workspace, size_t workspace_bytes, br_stream_t stream);
+                       float out_scale, void* workspace, size_t workspace_bytes, br_stream_t stream);
 
 /* br_hip_gelu_bwd (fp32) and br_hip_colsum_cast in one pass: dx = dy * gelu'(x)
  * is written as fp32 (dx may be x's or dy's own buffer), as a 16-bit copy dx16
@@ -144,7 +147,7 @@ int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int
  * separate entries.  BR_ERR_TODO unless cols % 4 == 0 and 16-byte aligned
  * operands; workspace as for br_hip_colsum. */
 int br_hip_gelu_bwd_colsum_cast(const float* dy, const float* x, float* dx, float* out, void* dx16,
-                                int dx16_dtype, int64_t rows, int64_t cols, void* workspace,
+                                int dx16_dtype, int64_t rows, int64_t cols, float out_scale, void* workspace,
                                 size_t workspace_bytes, br_stream_t stream);
 
 /* ---- LayerNorm --------------------------------------------------------- */
@@ -167,12 +170,14 @@ int br_hip_layernorm_fwd_copy16(const float* x, const float* gamma, const float*
 
 /* kernels::launch_ln_bw_float, kernels/normalize_kernels.cu:361-383
  * (declared kernels/kernels.h:28) with means == nullptr, called at cuda_tensor.cpp:699-727.  y is the forward
- * OUTPUT, var what the forward stored; dgamma / dbeta are overwritten. */
+ * OUTPUT, var what the forward stored; dgamma / dbeta are overwritten with
+ * the sums times param_scale (1, or 1/S when dy carries a power-of-two lift S
+ * that dx keeps and the parameter gradients must not). */
 size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols);
 int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma,
                          const float* beta, const float* var, float* dgamma, float* dbeta,
-                         float* dx, int64_t rows, int64_t cols, float eps, void* workspace,
-                         size_t workspace_bytes, br_stream_t stream);
+                         float* dx, int64_t rows, int64_t cols, float eps, float param_scale,
+                         void* workspace, size_t workspace_bytes, br_stream_t stream);
 
 /* The same backward with a residual gradient added to the input gradient:
  * dx = layernorm_backward(...) + residual, the `op.layernorm_backward` +
@@ -183,8 +188,8 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma,
 int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* gamma,
                                   const float* beta, const float* var, const float* residual,
                                   float* dgamma, float* dbeta, float* dx, int64_t rows,
-                                  int64_t cols, float eps, void* workspace, size_t workspace_bytes,
-                                  br_stream_t stream);
+                                  int64_t cols, float eps, float param_scale, void* workspace,
+                                  size_t workspace_bytes, br_stream_t stream);
 
 /* ---- softmax family ---------------------------------------------------- */
 /* cudnnSoftmaxForward(ACCURATE, INSTANCE) at cuda_tensor.cpp:332-356 and
@@ -374,13 +379,13 @@ int br_hip_probe_mfma_f16(int random_operands, int passes, float* scratch, int64
 /* The embedding row gather of blackriver/train_bloom.cpp:50-56. */
 int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, int elem_bytes,
                             int64_t n, int64_t hidden, int64_t vocab, br_stream_t stream);
-/* Backward of that gather: grad[ids[i], :] += dx[i, :] for i = 0 .. n-1 in
+/* Backward of that gather: grad[ids[i], :] += dx_scale * dx[i, :] for i = 0 .. n-1 in
  * ascending i (fp32; repeated ids are summed in position order, so the result
  * is deterministic); ids outside [0, vocab) are skipped.  The reference has no
  * embedding gradient (its table is frozen, train.words:264-268 only gathers);
  * with the LM head tied to the table this completes the table's gradient. */
 int br_hip_embedding_scatter_add(const float* dx, const int32_t* ids, float* grad, int64_t n,
-                                 int64_t hidden, int64_t vocab, br_stream_t stream);
+                                 int64_t hidden, int64_t vocab, float dx_scale, br_stream_t stream);
 /* The ALiBi table of train_bloom.cpp:58-71: alibi[h,k] = (float)(k*slope_h),
  * slope_h = (2^(-2^(3-log2 heads)))^(h+1) evaluated in fp64 on the host. */
 int br_hip_alibi_table(float* alibi, int64_t heads, int64_t tokens, br_stream_t stream);

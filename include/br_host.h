@@ -106,6 +106,13 @@ int br_bloom_model_create(br_env_t* env, int layers, int64_t batch, int64_t toke
 int br_bloom_model_set_fused_attention(br_env_t* env, int on);
 int br_bloom_model_init(br_env_t* env, uint64_t seed, float std);
 int br_bloom_model_step(br_env_t* env, const int32_t* ids, const int32_t* mask, float* loss);
+/* The power of two S that the last step's backward pass carried on its
+ * activation gradients (chosen by the loss head when products run in 16 bit so
+ * that small gradients stay clear of fp16's subnormal range; 1 with fp32
+ * products).  Parameter gradients are at their true scale; activation-gradient
+ * buffers left behind (e.g. `xc`, the embedding rows' gradient) hold S times
+ * the true values. */
+int br_bloom_model_grad_lift(br_env_t* env, float* lift);
 /* AdamW over every parameter of the model (the reference's loop ends at the
  * gradients, bloomz-7b/train.words:320-366).  optimizer_create allocates the
  * moments and, for 16-bit matrices, fp32 master copies initialised from the

@@ -27,7 +27,7 @@ def setup_block(runtime, hidden, heads, batch, tokens, mode, vocab=1024, seed=3)
     env.execute("%d %d %d 1e-05 model_dims" % (hidden, heads, vocab))
     env.set("$DEVICE", "cuda")
     env.set("$WDTYPE", {"f16": "f16", "bf16": "bf16"}.get(mode, "float"))
-    env.execute("'%s' op.gemm_precision" % {"f16": "f16", "bf16": "bf16"}.get(mode, "f32"))
+    env.execute("'%s' op.gemm_precision  1 op.grad_lift" % {"f16": "f16", "bf16": "bf16"}.get(mode, "f32"))
     env.execute("create_layer_weight create_layer_grad zero_layer_grad")
     env.execute("%d %d dynamic_floats" % (batch, tokens))
     floats = int(env.pop_number()) + 64 * vocab
@@ -203,6 +203,47 @@ def test_loss_head_at_the_true_vocabulary_keeps_small_probabilities(runtime):
     err = np.linalg.norm(wg[rare] - ref_rows, axis=1) / np.linalg.norm(ref_rows, axis=1)
     assert float(err.max()) <= 2e-2, "rare-token rows of lm_head_g: worst relative row error %.3g" % float(err.max())
     env.close()
+
+
+def test_gradient_lift_scales_activation_gradients_only(runtime):
+    """`S op.grad_lift`: the loss head hands out S * x_g, the block's backward
+    passes the factor on and takes it out of every parameter gradient.  With
+    fp32 products a power-of-two S commutes with every rounding, so parameter
+    gradients equal the unlifted run's bit for bit and activation gradients are
+    exactly S times as large; `0 op.grad_lift` picks S from the loss count only
+    when products run in 16 bit."""
+    hidden, heads, batch, tokens, vocab = 256, 4, 2, 24, 512
+    env, _, x, dy, mask, ids = setup_block(runtime, hidden, heads, batch, tokens, "fp32", vocab=vocab)
+    try:
+        rng = np.random.default_rng(21)
+        lm = (0.05 * rng.standard_normal((vocab, hidden))).astype(np.float32)
+        env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight' !" % (vocab, hidden))
+        env.execute("%d %d 2 'cuda' 'float' op.create 'lm_head.weight_g' !" % (vocab, hidden))
+        env.write("lm_head.weight", lm)
+        names = [n + "_g" for n in blk.WEIGHT_NAMES] + ["lm_head.weight_g"]
+        step = ("'lm_head.weight_g' @ op.zero  layer_forward  'xa' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ "
+                "'yout_g' @ 'lm_head.weight_g' @ op.loss_backward  layer_backward_core op.sync")
+        env.execute(step)
+        plain = {n: env.read(n) for n in names + ["xa"]}
+        env.write("xinput", x)
+        env.execute("256 op.grad_lift  bloom.grad_lift")
+        assert env.pop_number() == 256.0
+        env.execute(step)
+        for n in names:
+            assert np.array_equal(env.read(n), plain[n]), n
+        assert np.array_equal(env.read("xa"), plain["xa"] * np.float32(256)), "dx carries the lift"
+        # choosing per step: fp32 products need no lift
+        env.write("xinput", x)
+        env.execute("0 op.grad_lift")
+        env.execute(step)
+        env.execute("bloom.grad_lift")
+        assert env.pop_number() == 1.0
+        assert np.array_equal(env.read("xa"), plain["xa"])
+        with pytest.raises(host.HostError, match="power of two"):
+            env.execute("3 op.grad_lift")
+    finally:
+        env.execute("1 op.grad_lift")
+        env.close()
 
 
 def test_loss_value_and_chunking(runtime, capfd):

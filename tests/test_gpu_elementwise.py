@@ -133,7 +133,7 @@ def test_colsum(rows, cols):
     x = rng.standard_normal((rows, cols)).astype(np.float32)
     out = empty(cols)
     ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
-    call("br_hip_colsum", ptr(dev(x)), F32, ptr(out), rows, cols, ptr(ws), ws.numel(), stream())
+    call("br_hip_colsum", ptr(dev(x)), F32, ptr(out), rows, cols, 1.0, ptr(ws), ws.numel(), stream())
     assert_close(host(out), x.astype(np.float64).sum(0), RTOL, "colsum")
 
 
@@ -146,8 +146,8 @@ def test_colsum_cast_equals_colsum_plus_cast(rows, cols):
     dx = dev(x)
     ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
     sums, sums2, h = empty(cols), empty(cols), empty((rows, cols), torch.float16)
-    call("br_hip_colsum", ptr(dx), F32, ptr(sums), rows, cols, ptr(ws), ws.numel(), stream())
-    call("br_hip_colsum_cast", ptr(dx), ptr(sums2), ptr(h), F16, rows, cols, ptr(ws), ws.numel(), stream())
+    call("br_hip_colsum", ptr(dx), F32, ptr(sums), rows, cols, 1.0, ptr(ws), ws.numel(), stream())
+    call("br_hip_colsum_cast", ptr(dx), ptr(sums2), ptr(h), F16, rows, cols, 1.0, ptr(ws), ws.numel(), stream())
     assert np.array_equal(host(sums2), host(sums))
     assert np.array_equal(host(h).view(np.uint16), x.astype(np.float16).view(np.uint16))
     assert_close(host(sums2), x.astype(np.float64).sum(0), RTOL, "colsum")
@@ -266,7 +266,7 @@ def test_embedding_scatter_add_is_the_sequential_scatter(n, hidden, vocab):
     grad = rng.standard_normal((vocab, hidden)).astype(np.float32)
     want = orc.embedding_scatter_add(grad, dx, ids)
     d_grad = dev(grad)
-    call("br_hip_embedding_scatter_add", ptr(dev(dx)), ptr(dev(ids)), ptr(d_grad), n, hidden, vocab, stream())
+    call("br_hip_embedding_scatter_add", ptr(dev(dx)), ptr(dev(ids)), ptr(d_grad), n, hidden, vocab, 1.0, stream())
     assert np.array_equal(host(d_grad), want)
 
 
@@ -345,16 +345,16 @@ def test_gelu_bwd_colsum_cast_equals_the_separate_kernels(rows, cols, dtype, tdt
     call("br_hip_gelu_bwd", ptr(d_dy), ptr(d_x), ptr(dx_sep), F32, n, stream())
     ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
     sums_sep, x16_sep = empty(cols), empty((rows, cols), tdtype)
-    call("br_hip_colsum_cast", ptr(dx_sep), ptr(sums_sep), ptr(x16_sep), dtype, rows, cols, ptr(ws), ws.numel(), stream())
+    call("br_hip_colsum_cast", ptr(dx_sep), ptr(sums_sep), ptr(x16_sep), dtype, rows, cols, 1.0, ptr(ws), ws.numel(), stream())
     for in_place in (False, True):
         d_u = dev(x)
         dx = d_u if in_place else empty((rows, cols))
         sums, x16 = empty(cols), empty((rows, cols), tdtype)
         call("br_hip_gelu_bwd_colsum_cast", ptr(d_dy), ptr(d_u), ptr(dx), ptr(sums), ptr(x16), dtype, rows, cols,
-             ptr(ws), ws.numel(), stream())
+             1.0, ptr(ws), ws.numel(), stream())
         assert torch.equal(dx, dx_sep), in_place
         assert torch.equal(x16.view(torch.int16), x16_sep.view(torch.int16)), in_place
         assert torch.equal(sums, sums_sep), in_place
     assert hip.load().br_hip_gelu_bwd_colsum_cast(ptr(d_dy), ptr(d_x), ptr(dx_sep), ptr(sums_sep), ptr(x16_sep), dtype,
-                                                  4, 1001, ptr(ws), ws.numel(), stream()) == -1
+                                                  4, 1001, 1.0, ptr(ws), ws.numel(), stream()) == -1
     torch.cuda.synchronize()

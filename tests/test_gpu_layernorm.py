@@ -29,13 +29,13 @@ def run_fwd(x, g, b, eps, offset=0):
     return host(y), host(mean), host(var)
 
 
-def run_bwd(dy, y, g, b, var, eps):
+def run_bwd(dy, y, g, b, var, eps, param_scale=1.0):
     rows, cols = dy.shape
     dgam, dbet, dx = empty(cols), empty(cols), empty((rows, cols))
     ws = workspace(hip.load().br_hip_layernorm_bwd_workspace(rows, cols))
     t = [dev(a) for a in (dy, y, g, b, var)]
     call("br_hip_layernorm_bwd", ptr(t[0]), ptr(t[1]), ptr(t[2]), ptr(t[3]), ptr(t[4]), ptr(dgam), ptr(dbet),
-         ptr(dx), rows, cols, eps, ptr(ws), ws.numel(), stream())
+         ptr(dx), rows, cols, eps, param_scale, ptr(ws), ws.numel(), stream())
     return host(dx), host(dgam), host(dbet)
 
 
@@ -97,7 +97,7 @@ def test_layernorm_rejects_bad_arguments():
     assert lib.br_hip_layernorm_fwd(ptr(t), ptr(t), ptr(t), None, None, None, 1, 16, 1e-5, stream()) == -3
     assert lib.br_hip_layernorm_fwd(ptr(t), ptr(t), ptr(t), ptr(t), None, None, 1, 0, 1e-5, stream()) == -4
     assert lib.br_hip_layernorm_bwd(ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 1, 16, 1e-5,
-                                    None, 0, stream()) == -4
+                                    1.0, None, 0, stream()) == -4
     torch.cuda.synchronize()
 
 
@@ -156,12 +156,29 @@ def test_layernorm_bwd_with_residual_equals_backward_then_add(rows, cols):
         dgam, dbet = empty(cols), empty(cols)
         out = {"none": empty((rows, cols)), "residual": t_res, "dy": t_dy}[alias]
         call("br_hip_layernorm_bwd_residual", ptr(t_dy), ptr(t_y), ptr(t_g), ptr(t_b), ptr(t_var), ptr(t_res),
-             ptr(dgam), ptr(dbet), ptr(out), rows, cols, eps, ptr(ws), ws.numel(), stream())
+             ptr(dgam), ptr(dbet), ptr(out), rows, cols, eps, 1.0, ptr(ws), ws.numel(), stream())
         assert np.array_equal(host(out), want), alias
         assert np.array_equal(host(dgam), dg_plain) and np.array_equal(host(dbet), db_plain), alias
     # shapes the row kernel cannot take are declined
     t = empty(4 * 1001)
     gg = empty(1001)
     assert hip.load().br_hip_layernorm_bwd_residual(ptr(t), ptr(t), ptr(gg), ptr(gg), ptr(gg), ptr(t), ptr(gg), ptr(gg),
-                                                    ptr(t), 4, 1001, eps, ptr(ws), ws.numel(), stream()) == -1
+                                                    ptr(t), 4, 1001, eps, 1.0, ptr(ws), ws.numel(), stream()) == -1
     torch.cuda.synchronize()
+
+
+def test_layernorm_bwd_param_scale_is_an_exact_power_of_two_factor():
+    """dy lifted by S = 1024 with param_scale = 1/S: dx comes out S times the
+    plain one and dgamma / dbeta equal the plain ones, all bit for bit (scaling
+    by a power of two commutes with every rounding on the way)."""
+    rng = np.random.default_rng(31)
+    rows, cols, eps = 96, 1024, 1e-5
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    g = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    b = (0.1 * rng.standard_normal(cols)).astype(np.float32)
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    y, _, var = run_fwd(x, g, b, eps)
+    dx, dg, db = run_bwd(dy, y, g, b, var, eps)
+    dx2, dg2, db2 = run_bwd(dy * np.float32(1024), y, g, b, var, eps, param_scale=1.0 / 1024)
+    assert np.array_equal(dx2, dx * np.float32(1024))
+    assert np.array_equal(dg2, dg) and np.array_equal(db2, db)

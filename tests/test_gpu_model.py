@@ -23,12 +23,12 @@ MODEL_NAMES = ["word_embeddings.weight", "word_embeddings_layernorm.weight", "wo
                "ln_f.weight", "ln_f.bias"]
 
 
-def build(mode, layers, batch, tokens, hidden, heads, vocab, seed):
+def build(mode, layers, batch, tokens, hidden, heads, vocab, seed, std=0.05):
     rng = np.random.default_rng(seed)
     wdtype = {"f16": "f16", "bf16": "bf16"}.get(mode, "float")
     model = host.BloomModel(layers, batch, tokens, hidden, heads, vocab, 1e-5, wdtype,
                             wdtype if wdtype != "float" else "f32")
-    model.init(seed, 0.05)
+    model.init(seed, std)
     # LayerNorm parameters and biases away from their 1 / 0 defaults
     for i in range(1, layers + 1):
         for name in ("input_layernorm", "post_attention_layernorm"):
@@ -59,14 +59,17 @@ def build(mode, layers, batch, tokens, hidden, heads, vocab, seed):
 ])
 def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden, heads, vocab):
     print("case %s layers=%d batch=%d tokens=%d hidden=%d" % (mode, layers, batch, tokens, hidden), flush=True)
-    model, model_w, layer_ws, ids, mask = build(mode, layers, batch, tokens, hidden, heads, vocab, seed=7)
+    # the full-width case takes config C5's N(0, 0.02) matrices; at hidden 4096 a standard deviation of 0.05
+    # gives attention scores of +-10 and probabilities whose fp16-operand error alone exceeds the bound
+    std = 0.02 if hidden >= 4096 else 0.05
+    model, model_w, layer_ws, ids, mask = build(mode, layers, batch, tokens, hidden, heads, vocab, seed=7, std=std)
     # bf16: one block holds 6e-2 (tests/test_gpu_block.py); two blocks, the head and the tied
     # table's gradient (a sum of two bf16-product results) compound to just under 1e-1
     tol = {"fp32": 2e-4, "f16": 2e-2, "bf16": 1e-1}[mode]
     try:
         # different initial matrices per block (a seed slip would make them equal)
         assert not np.array_equal(layer_ws[0]["dense.weight"], layer_ws[1]["dense.weight"])
-        assert 0.03 < float(np.std(layer_ws[0]["dense_h_to_4h.weight"])) < 0.07
+        assert 0.6 * std < float(np.std(layer_ws[0]["dense_h_to_4h.weight"])) < 1.4 * std
         loss = model.step(ids, mask)
         ref_loss, ref = mdl.model_step(model_w, layer_ws, ids, mask, heads, 1e-5)
         assert abs(loss - ref_loss) <= tol * abs(ref_loss), (loss, ref_loss)
@@ -75,10 +78,23 @@ def test_model_step_matches_oracle(runtime, mode, layers, batch, tokens, hidden,
                 if name == "key.bias":      # zero up to rounding (softmax shift invariance)
                     continue
                 assert_close(model.read(i, name + "_g"), ref[i][name + "_g"], tol, "block %d %s_g" % (i, name))
-        for name in ("ln_f.weight", "ln_f.bias", "word_embeddings_layernorm.weight",
-                     "word_embeddings_layernorm.bias", "word_embeddings.weight"):
+        for name in ("ln_f.weight", "ln_f.bias", "word_embeddings_layernorm.weight", "word_embeddings_layernorm.bias"):
             assert_close(model.read(0, name + "_g"), ref[0][name + "_g"], tol, name + "_g")
-        assert_close(model.read(0, "xc"), ref[0]["embedding_rows_g"], tol, "gradient of the embedding rows")
+        # The tied table's gradient: rows of the batch's ids (the scattered embedding-row gradients on top
+        # of the head's) and all other rows (the head's alone) are held to the bound separately, each
+        # against its own scale -- at 250880 rows the rms of the whole table says nothing about the
+        # few hundred rows the scatter touches.
+        table, table_ref = model.read(0, "word_embeddings.weight_g"), ref[0]["word_embeddings.weight_g"]
+        touched = np.zeros(vocab, bool)
+        touched[ids.reshape(-1)] = True
+        assert_close(table[touched], table_ref[touched], tol, "word_embeddings.weight_g, rows of the batch")
+        assert_close(table[~touched], table_ref[~touched], tol, "word_embeddings.weight_g, other rows")
+        del table, table_ref
+        # activation gradients are left carrying the step's gradient lift (a power of two; 1 in fp32 mode)
+        lift = model.grad_lift()
+        assert lift == (1.0 if mode == "fp32" else 16.0 * 2 ** int(np.ceil(np.log2(orc.loss_labels(ids, mask)[1]))))
+        assert_close(model.read(0, "xc") / np.float32(lift), ref[0]["embedding_rows_g"], tol,
+                     "gradient of the embedding rows")
         # the head is tied to the table: one gradient tensor under both names
         assert np.array_equal(model.read(0, "lm_head.weight_g"), model.read(0, "word_embeddings.weight_g"))
         # a second step on the same batch: gradients are overwritten, the head's
