@@ -9,6 +9,8 @@
 // beta and running dgamma / dbeta sums for its own columns in registers, so
 // dy and y are read exactly once; per-workgroup partial column sums go to a
 // workspace and a small second kernel adds them in a fixed order.
+#include <mutex>
+
 #include "common.hpp"
 
 #include <stdlib.h>
@@ -374,6 +376,38 @@ int layernorm_fwd_launch(const float* x, const float* gamma, const float* beta, 
 }
 }  // namespace
 
+// ---- scratch of the entry point that allocates nothing ---------------------
+// Partial sums go to a file-scope device array instead of a caller workspace.
+// Every GPU the library runs on holds its own copy of the array (until the
+// process ends) at its own address; the address is looked up once per device,
+// with that device current, and only that pointer is ever handed to kernels.
+// (No `used` attribute on the array: with it the compiler keeps the symbol
+// internal to the code object and the runtime's lookup by name cannot find it.)
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device; hipError_t on failure.
+int static_scratch(void** out) {
+    int dev = -1;
+    BR_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return BR_ERR_ATTR;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        BR_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return BR_OK;
+}
+}  // namespace
+
 extern "C" {
 
 int br_hip_layernorm_fwd(const float* x, const float* gamma, const float* beta, float* y, float* mean,
@@ -470,6 +504,24 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma, co
                          float eps, float param_scale, void* workspace, size_t workspace_bytes, br_stream_t stream) {
     return layernorm_bwd_impl(dy, y, gamma, beta, var, nullptr, dgamma, dbeta, dx, rows, cols, eps, param_scale,
                               workspace, workspace_bytes, stream);
+}
+
+// ---- the entry point that allocates nothing -------------------------------
+size_t br_hip_layernorm_bwd_static_limit(void) { return kStaticScratchBytes; }
+
+int br_hip_layernorm_bwd_static(const float* dy, const float* y, const float* gamma, const float* beta,
+                                const float* var, float* dgamma, float* dbeta, float* dx, int64_t rows, int64_t cols,
+                                float eps, float param_scale, br_stream_t stream) {
+    if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
+    const size_t need = br_hip_layernorm_bwd_workspace(rows, cols);
+    if (need > kStaticScratchBytes) return BR_ERR_SCRATCH;
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != BR_OK) return rc;
+    // every partial the finalize pass reads is written by the main pass of the
+    // same call, so nothing in the array has to start at zero
+    return layernorm_bwd_impl(dy, y, gamma, beta, var, nullptr, dgamma, dbeta, dx, rows, cols, eps, param_scale, ws,
+                              kStaticScratchBytes, stream);
 }
 
 int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* gamma, const float* beta,

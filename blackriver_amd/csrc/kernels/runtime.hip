@@ -47,6 +47,7 @@ const char* br_hip_error_string(int code) {
         case BR_ERR_INPUT: return "br_hip: bad input argument";
         case BR_ERR_OUTPUT: return "br_hip: bad output argument";
         case BR_ERR_ATTR: return "br_hip: bad attribute or size";
+        case BR_ERR_SCRATCH: return "br_hip: problem too large for the built-in scratch buffer of an allocation-free entry";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);

@@ -62,6 +62,8 @@ SIGNATURES = {
     "br_hip_layernorm_fwd_copy16": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _vp, _vp, _i64, _i64, _f32, _vp]),
     "br_hip_layernorm_bwd_workspace": (_sz, [_i64, _i64]),
     "br_hip_layernorm_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _f32, _vp, _sz, _vp]),
+    "br_hip_layernorm_bwd_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _f32, _vp]),
+    "br_hip_layernorm_bwd_static_limit": (_sz, []),
     "br_hip_layernorm_bwd_residual": (_int, [_vp] * 9 + [_i64, _i64, _f32, _f32, _vp, _sz, _vp]),
     "br_hip_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "br_hip_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),

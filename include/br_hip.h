@@ -8,7 +8,8 @@
  * positive hipError_t value when the HIP runtime failed, or a negative
  * BR_ERR_* value when the arguments are rejected before any launch.  Nothing
  * here allocates device memory except br_hip_malloc / br_hip_host_malloc;
- * kernels that need scratch take a caller-provided workspace.
+ * kernels that need scratch take a caller-provided workspace (one entry,
+ * br_hip_layernorm_bwd_static, uses a buffer built into the library instead).
  *
  * Tensors are dense row-major.  "dtype" arguments use the numbering of the
  * reference's br::DataType (blackriver/tensortype.hpp:16-21).
@@ -41,7 +42,9 @@ enum {
     BR_ERR_TODO = -1,     /* combination not implemented  (OP_TODO_ERROR)   */
     BR_ERR_INPUT = -2,    /* bad input argument           (OP_INPUT_ERROR)  */
     BR_ERR_OUTPUT = -3,   /* bad output argument          (OP_OUTPUT_ERROR) */
-    BR_ERR_ATTR = -4      /* bad scalar attribute / size  (OP_ATTR_ERROR)   */
+    BR_ERR_ATTR = -4,     /* bad scalar attribute / size  (OP_ATTR_ERROR)   */
+    BR_ERR_SCRATCH = -5   /* problem needs more scratch than the library's
+                             built-in buffer holds (allocation-free entries) */
 };
 
 /* ---- runtime plumbing -------------------------------------------------- */
@@ -178,6 +181,23 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma,
                          const float* beta, const float* var, float* dgamma, float* dbeta,
                          float* dx, int64_t rows, int64_t cols, float eps, float param_scale,
                          void* workspace, size_t workspace_bytes, br_stream_t stream);
+
+/* br_hip_layernorm_bwd without the workspace argument, for callers that cannot
+ * allocate device memory or hand a workspace in: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+ * in the reference.  The partial sums go to a buffer built into the library
+ * (br_hip_layernorm_bwd_static_limit() bytes, 16 MiB, held once per GPU for the
+ * life of the process); the call makes no hipMalloc / hipFree and uses the
+ * same kernels as br_hip_layernorm_bwd, so results are identical bit for bit.
+ * Returns BR_ERR_SCRATCH when br_hip_layernorm_bwd_workspace(rows, cols)
+ * exceeds the limit (e.g. cols > 4096 at 512 or more rows).  All calls on one
+ * GPU share the buffer: calls that overlap in time on one GPU (two streams)
+ * race; calls on one stream, or ordered by events, are safe. */
+size_t br_hip_layernorm_bwd_static_limit(void);
+int br_hip_layernorm_bwd_static(const float* dy, const float* y, const float* gamma,
+                                const float* beta, const float* var, float* dgamma, float* dbeta,
+                                float* dx, int64_t rows, int64_t cols, float eps, float param_scale,
+                                br_stream_t stream);
 
 /* The same backward with a residual gradient added to the input gradient:
  * dx = layernorm_backward(...) + residual, the `op.layernorm_backward` +
