@@ -54,7 +54,11 @@ namespace gemm16 {
 typedef __attribute__((address_space(3))) unsigned char lds_byte;
 
 // One wave-wide direct-to-LDS load: lane l copies the 16 bytes at
-// sbase + voff(l) to LDS byte lds_dst + 16*l.
+// sbase + voff(l) to LDS byte lds_dst + 16*l.  M0 is written inside the
+// statement and not named as clobbered: the compiler treats M0 as reserved and
+// rejects it in a clobber list; it holds no compiler-owned value here because
+// these kernels contain none of the operations the compiler itself routes
+// through M0 (indexed register moves, GWS, messages, lane-indexed reads).
 __device__ __forceinline__ void dtl_load(unsigned lds_dst, unsigned voff, const void* sbase) {
     asm volatile(
         "s_mov_b32 m0, %0\n\t"
@@ -147,6 +151,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     constexpr int kLoads = TA::kPerWave + TB::kPerWave;  // per wave and tile
     static_assert(STAGES >= 2 && STAGES <= 4, "two to four tile buffers");
     static_assert(KT == 32 || KT == 64, "K tile of 32 or 64");
+    static_assert(FM * FN >= FM + FN, "one LDS fragment read per MFMA slot");
     static_assert(STAGES * kStageBytes <= 160 * 1024, "LDS");
     __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[STAGES * kStageBytes];
     const lds_byte* lds = (const lds_byte*)lds_raw;
@@ -208,11 +213,25 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
         for (int j = 0; j < FN; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
-    auto multiply = [&](const u32x4 (&fa)[FM], const u32x4 (&fb)[FN]) {
+    // One sub-step, in the instruction order the hardware is to see: the MFMAs of
+    // the fragments in hand (fa, fb), with the LDS reads that fetch the next
+    // sub-step's fragments (na, nb; from `tile`, sub-step `ks`) slotted in one
+    // per MFMA.  The scheduling fences pin that order: left alone, the compiler
+    // sinks the reads below the MFMAs to reuse their registers, and the next
+    // sub-step's first MFMA then waits out the full LDS latency.
+    auto step = [&](const u32x4 (&fa)[FM], const u32x4 (&fb)[FN], u32x4 (&na)[FM], u32x4 (&nb)[FN], int tile, int ks) {
+        const lds_byte* stage = lds + (tile % STAGES) * kStageBytes;
 #pragma unroll
-        for (int i = 0; i < FM; i++)
-#pragma unroll
-            for (int j = 0; j < FN; j++) acc[i][j] = Cvt<CT>::mfma(fa[i], fb[j], acc[i][j]);
+        for (int idx = 0; idx < FM * FN; idx++) {
+            // column-major walk over the wave's blocks: the first FM MFMAs need only fb[0];
+            // fragments are fetched in the order the next sub-step uses them: fb[0], fa[0..], fb[1..]
+            const int i = idx % FM, j = idx / FM;
+            if (idx == 0) nb[0] = TB::fragment(stage, fb_off[0][ks]);
+            else if (idx <= FM) na[idx - 1] = TA::fragment(stage, fa_off[idx - 1][ks]);
+            else if (idx < FM + FN) nb[idx - FM] = TB::fragment(stage, fb_off[idx - FM][ks]);
+            acc[i][j] = Cvt<CT>::mfma(fa[i], fb[j], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     };
 
     // Fill the ring, wait for tile 0 and read its first sub-step of fragments.
@@ -229,7 +248,11 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     // the next sub-step are in flight.
     u32x4 fa0[FM], fb0[FN], fa1[FM], fb1[FN];
     read_frags(fa0, fb0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
 
+    // The MFMA stream is free of branches: the last tile's final sub-step also
+    // fetches (from the buffer a tile nk would occupy; the values are never
+    // used) and passes the barrier like every other.
     for (int t = 0; t < nk; t++) {
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
@@ -238,8 +261,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
             u32x4(&fa_next)[FM] = (ks & 1) ? fa0 : fa1;
             u32x4(&fb_next)[FN] = (ks & 1) ? fb0 : fb1;
             if (ks + 1 < KS) {
-                read_frags(fa_next, fb_next, t, ks + 1);
-            } else if (t + 1 < nk) {
+                step(fa_now, fb_now, fa_next, fb_next, t, ks + 1);
+            } else {
                 // tile t+1 has to be in LDS; the tiles issued after it may stay in flight
                 const int after = nk - 2 - t;
                 if (after >= STAGES - 2) {
@@ -252,9 +275,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                 // every wave has now read all of tile t, so its buffer can be refilled
                 __syncthreads();
                 if (t + STAGES < nk) issue(t + STAGES);
-                read_frags(fa_next, fb_next, t + 1, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                step(fa_now, fb_now, fa_next, fb_next, t + 1, 0);
             }
-            multiply(fa_now, fb_now);
         }
     }
 
@@ -353,6 +376,8 @@ int launch_dtl(const GemmArgs& g, const Problem& p, long long batch, hipStream_t
     if (pick != 3 && force && strcmp(force, "256x256") == 0) pick = 0;
     if (pick != 3 && force && strcmp(force, "256x128") == 0) pick = 1;
     if (pick != 3 && force && strcmp(force, "128x128") == 0) pick = 2;
+    if (pick == 0 && force && strcmp(force, "256x256w4") == 0)
+        return launch_dtl_config<CT, 256, 256, 128, 128, 64, 2>(g, p, batch, st);
     if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
     if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
     if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
