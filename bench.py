@@ -279,7 +279,7 @@ def elementwise_leg(hip, timer, torch):
     rec("bias_gelu_fwd [2048,16384] f16", sec, 2 * rows * cols * 2)
     ws = torch.empty(lib.br_hip_bias_gelu_bwd_workspace(rows, cols), dtype=torch.uint8, device="cuda")
     sec = timer.run(lambda i: hip.call("br_hip_bias_gelu_bwd", vp(dys[i % nb]), vp(xs[i % nb]), vp(bias), vp(ys[i % nb]),
-                                       vp(dbias), hip.F16, rows, cols, vp(ws), ws.numel(), st), 200, 10)
+                                       vp(dbias), hip.F16, rows, cols, 1.0, vp(ws), ws.numel(), st), 200, 10)
     rec("bias_gelu_bwd [2048,16384] f16 (+dbias)", sec, 3 * rows * cols * 2)
     del xs, ys, dys
 

@@ -742,9 +742,54 @@ ComputingReturn hip_gelu_linear_backward(const tensor_t& dy, const tensor_t& u, 
             }
         }
     }
+    // everything already in the products' 16-bit type (the 4h activation and its gradient kept in the
+    // products' type): one pass gives du and the bias gradient, du is the
+    // products' operand as it stands
+    const DataType gdt = dy->dtype();
+    const bool half = dev(dy) && dev(u) && dev(du) && (gdt == DataType::F16 || gdt == DataType::BF16) &&
+                      u->dtype() == gdt && du->dtype() == gdt && dev(x) && dev(weight) && dev(x_g) && dev(weight_g) &&
+                      dev_f32(bias_g) && du->shape().dim() == 3 && x->shape().dim() == 3 &&
+                      u->items() == dy->items() && du->items() == dy->items();
+    if (half) {
+        const int64_t n = (int64_t)(du->shape()[0] * du->shape()[1]);
+        const int64_t out = (int64_t)du->shape()[2], in = (int64_t)x->shape()[2];
+        const int compute = pick_compute({du, x, weight});
+        const int native = compute == BR_GEMM_F16 ? BR_F16 : compute == BR_GEMM_BF16 ? BR_BF16 : BR_F32;
+        if (native == (int)gdt && out % 8 == 0 && (int64_t)x->items() == n * in && (int64_t)weight->items() == out * in &&
+            (int64_t)x_g->items() == n * in && (int64_t)weight_g->items() == out * in &&
+            (int64_t)bias_g->items() == out) {
+            const size_t need = br_hip_bias_gelu_bwd_workspace(n, out);
+            void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
+            BR_OP(br_hip_bias_gelu_bwd(dy->data(), u->data(), nullptr, du->data(), static_cast<float*>(bias_g->data()),
+                                       native, n, out, unlift(), ws, need, stream()));
+            BR_OP(linear_backward_products(Operand{du->data(), native}, x, weight, x_g, weight_g, n, in, out, compute));
+            return OP_OK;
+        }
+    }
     ComputingReturn r = dy->op_gelu_backward(dy, u, du);
     if (r != OP_OK) return r;
     return du->op_linear_backward(du, x, weight, bias, x_g, weight_g, bias_g);
+}
+
+ComputingReturn hip_linear_gelu(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& u,
+                                const tensor_t& y) {
+    if (!dev(x) || !dev(w) || !dev(bias) || x->shape().dim() != 3) return OP_INPUT_ERROR;
+    if (!dev(u) || !dev(y) || u->items() != y->items() || u->data() == y->data()) return OP_OUTPUT_ERROR;
+    const int64_t n = (int64_t)(x->shape()[0] * x->shape()[1]);
+    const int64_t in = (int64_t)x->shape()[2];
+    const int64_t out = (int64_t)w->shape()[0];
+    if ((int64_t)w->shape()[1] != in || (int64_t)bias->items() != out) return OP_INPUT_ERROR;
+    if ((int64_t)u->items() != n * out) return OP_OUTPUT_ERROR;
+    const DataType dt = x->dtype();
+    if ((dt == DataType::F16 || dt == DataType::BF16) && w->dtype() == dt && u->dtype() == dt && y->dtype() == dt) {
+        const int rc = br_hip_linear_gelu(x->data(), w->data(), bias_f32(bias, 0), u->data(), y->data(), (int)dt, n, out,
+                                          in, stream());
+        if (rc != BR_ERR_TODO) return done(rc, "br_hip_linear_gelu");
+    }
+    // the two operators
+    ComputingReturn r = x->op_linear(x, w, bias, u);
+    if (r != OP_OK) return r;
+    return u->op_gelu(u, y);
 }
 
 ComputingReturn hip_linear_accumulate(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& y) {

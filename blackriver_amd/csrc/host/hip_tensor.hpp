@@ -77,6 +77,11 @@ private:
 ComputingReturn hip_gelu_linear_backward(const tensor_t& dy, const tensor_t& u, const tensor_t& du, const tensor_t& x,
                                          const tensor_t& weight, const tensor_t& bias, const tensor_t& x_g,
                                          const tensor_t& weight_g, const tensor_t& bias_g);
+// u = x . w^T + bias, y = gelu(u): op_linear (cuda_tensor.cpp:146-193) followed by
+// op_gelu (:400-412).  With 16-bit tensors throughout, one product whose
+// epilogue writes both (gelu of the fp32 sum); otherwise the two operators.
+ComputingReturn hip_linear_gelu(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& u,
+                                const tensor_t& y);
 // y += x . w^T + bias: op_linear (cuda_tensor.cpp:146-193) followed by
 // op_add(y, ., y) with the addition done in the product's epilogue; the sum is
 // formed from the same fp32 values, so the bits equal the two operators'.

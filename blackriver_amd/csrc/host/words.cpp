@@ -369,6 +369,11 @@ BR_WORD(GeluLinearBackward,
         l[0]->op_linear_backward(l[0], l[1], l[2], l[3], l[4], l[5], l[6]);
     }
 )
+// ( x w b u y -- )   u = x . w^T + b,  y = gelu(u)      `op.linear` + `op.gelu`
+BR_WORD(LinearGelu,
+    Tensors<5> a(stack);
+    op_check_word(hip_linear_gelu(a[0], a[1], a[2], a[3], a[4]), "op.linear_gelu");
+)
 // ( x w b y -- )   y += x . w^T + b          `op.linear` into a temporary + `op.add`
 BR_WORD(LinearAdd,
     Tensors<4> a(stack);
@@ -469,6 +474,7 @@ void load_nn_words(Enviroment& env) {
         {"op.qk_backward", QueryKeyBackward::creator},
         {"op.gelu_linear_backward", GeluLinearBackward::creator},
         {"op.linear_add", LinearAdd::creator},
+        {"op.linear_gelu", LinearGelu::creator},
         {"op.layernorm_backward_add", LayernormBackwardAdd::creator},
         {"op.flash_attn", FlashAttn::creator},
         {"op.flash_attn_backward", FlashAttnBackward::creator},

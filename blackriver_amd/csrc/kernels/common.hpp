@@ -122,6 +122,16 @@ inline bool copy16_ok(const void* y16, int dtype) {
     return y16 && (dtype == BR_F16 || dtype == BR_BF16) && (reinterpret_cast<uintptr_t>(y16) & 7u) == 0;
 }
 
+// gelu(v) = v * (0.5 + 0.5*tanh(u)),  u = v*(0.79788456 + 0.03567741 v^2)
+//         = v * sigmoid(2u)            (no cancellation in the left tail)
+// sigmoid(2u) = 1 / (1 + 2^w), w = -2*log2(e)*u: the factor is folded into the
+// two polynomial constants, so the exponent costs no extra multiplies.
+constexpr float kLog2e2 = 2.8853900817779268f;  // 2 * log2(e)
+__device__ __forceinline__ float gelu_one(float v) {
+    const float w = v * (-kLog2e2 * 0.79788456f + (-kLog2e2 * 0.03567741f) * (v * v));
+    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(w));
+}
+
 // Grid size for a grid-stride elementwise kernel: enough workgroups to keep
 // 256 CUs busy several times over, never more than the work needs.
 inline int grid_for(int64_t work_items, int block, int max_blocks = 256 * 16) {

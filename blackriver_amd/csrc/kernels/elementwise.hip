@@ -190,16 +190,6 @@ __global__ __launch_bounds__(kBlock) void add_bcast_scalar(const T* a, const T* 
 }
 
 // ------------------------------------------------------------------ GELU
-// gelu(v) = v * (0.5 + 0.5*tanh(u)),  u = v*(0.79788456 + 0.03567741 v^2)
-//         = v * sigmoid(2u)            (no cancellation in the left tail)
-// sigmoid(2u) = 1 / (1 + 2^w), w = -2*log2(e)*u: the factor is folded into the
-// two polynomial constants, so the exponent costs no extra multiplies.
-constexpr float kLog2e2 = 2.8853900817779268f;  // 2 * log2(e)
-__device__ __forceinline__ float gelu_one(float v) {
-    const float w = v * (-kLog2e2 * 0.79788456f + (-kLog2e2 * 0.03567741f) * (v * v));
-    return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(w));
-}
-
 // d/dv gelu(v) = s + 2 v s (1 - s) u',  s = sigmoid(2u),
 //   u = 0.79788456 v (1 + 0.044715 v^2),  u' = 0.79788456 + 0.1070322243 v^2
 // evaluated from e = exp(-2|u|) = 2^(-|w|), w = 2*log2(e)*u, in (0,1] so that s
@@ -327,6 +317,38 @@ struct VecIO<__half, 8> {
         const half8 h = __builtin_bit_cast(half8, u);
         *reinterpret_cast<half8*>(p) = h;
         unpack8(h, f);
+    }
+};
+
+template <>
+struct VecIO<__hip_bfloat16, 8> {
+    static __device__ __forceinline__ void load(const __hip_bfloat16* p, float (&f)[8]) {
+        unpack(*reinterpret_cast<const uint4*>(p), f);
+    }
+    static __device__ __forceinline__ void unpack(const uint4& u, float (&f)[8]) {
+        const unsigned w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            f[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+            f[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ uint4 pack(const float (&f)[8]) {
+        unsigned w[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            w[i] = (unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(f[2 * i])) |
+                   ((unsigned)__builtin_bit_cast(unsigned short, __float2bfloat16(f[2 * i + 1])) << 16);
+        return make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    static __device__ __forceinline__ void store(__hip_bfloat16* p, const float (&f)[8]) {
+        *reinterpret_cast<uint4*>(p) = pack(f);
+    }
+    static __device__ __forceinline__ void store_rounded(__hip_bfloat16* p, float (&f)[8]) {
+        uint4 u = pack(f);
+        asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w));
+        *reinterpret_cast<uint4*>(p) = u;
+        unpack(u, f);
     }
 };
 
@@ -1003,13 +1025,13 @@ int br_hip_gelu_bwd(const void* dy, const void* x, void* dx, int dtype, int64_t 
 size_t br_hip_bias_gelu_bwd_workspace(int64_t rows, int64_t cols) { return br_hip_colsum_workspace(rows, cols); }
 
 int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void* dx, float* dbias, int dtype,
-                         int64_t rows, int64_t cols, void* workspace, size_t workspace_bytes,
+                         int64_t rows, int64_t cols, float dbias_scale, void* workspace, size_t workspace_bytes,
                          br_stream_t stream) {
     if (rows < 0 || cols <= 0) return BR_ERR_ATTR;
     if (rows == 0) return BR_OK;
     if (!dy || !x) return BR_ERR_INPUT;
     if (!dx) return BR_ERR_OUTPUT;
-    if (dtype != BR_F32 && dtype != BR_F16) return BR_ERR_TODO;
+    if (dtype != BR_F32 && dtype != BR_F16 && dtype != BR_BF16) return BR_ERR_TODO;
     hipStream_t st = as_stream(stream);
     const int rpb = strip_rows(rows);
     const int groups = (int)((rows + rpb - 1) / rpb);
@@ -1027,6 +1049,13 @@ int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void*
         dim3 grid((unsigned)((cols / 8 + kBlock - 1) / kBlock), (unsigned)groups);
         bias_gelu_bwd_kernel<__half, 8><<<grid, kBlock, 0, st>>>((const __half*)dy, (const __half*)x, bias,
                                                                   (__half*)dx, partial, rows, cols, rpb);
+    } else if (dtype == BR_BF16 && al && cols % 8 == 0) {
+        dim3 grid((unsigned)((cols / 8 + kBlock - 1) / kBlock), (unsigned)groups);
+        bias_gelu_bwd_kernel<__hip_bfloat16, 8><<<grid, kBlock, 0, st>>>((const __hip_bfloat16*)dy,
+                                                                         (const __hip_bfloat16*)x, bias,
+                                                                         (__hip_bfloat16*)dx, partial, rows, cols, rpb);
+    } else if (dtype == BR_BF16) {
+        return BR_ERR_TODO;
     } else {
         // unaligned shapes: elementwise pass, then a separate column sum of dx
         const int64_t n = rows * cols;
@@ -1037,11 +1066,11 @@ int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void*
             gelu_scalar<__half><<<grid_for(n, kBlock), kBlock, 0, st>>>((const __half*)dy, (const __half*)x,
                                                                        bias, (__half*)dx, n, cols, true);
         BR_HIP_LAUNCH_CHECK();
-        if (dbias) return br_hip_colsum(dx, dtype, dbias, rows, cols, 1.0f, workspace, workspace_bytes, stream);
+        if (dbias) return br_hip_colsum(dx, dtype, dbias, rows, cols, dbias_scale, workspace, workspace_bytes, stream);
         return BR_OK;
     }
     BR_HIP_LAUNCH_CHECK();
-    if (dbias) return colsum_finish(partial, dbias, groups, cols, 1.0f, st);
+    if (dbias) return colsum_finish(partial, dbias, groups, cols, dbias_scale, st);
     return BR_OK;
 }
 

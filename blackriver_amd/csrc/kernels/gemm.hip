@@ -254,6 +254,35 @@ extern "C" int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64
     return gemm16_launch_bf16(g, p, batch, st);
 }
 
+extern "C" int br_hip_linear_gelu(const void* x, const void* w, const float* bias, void* u, void* y, int dtype,
+                                  int64_t rows, int64_t out, int64_t in, br_stream_t stream) {
+    if (rows < 0 || out <= 0 || in <= 0) return BR_ERR_ATTR;
+    if (dtype != BR_F16 && dtype != BR_BF16) return BR_ERR_TODO;
+    if (rows == 0) return BR_OK;
+    if (!x || !w) return BR_ERR_INPUT;
+    if (!u || !y || u == y) return BR_ERR_OUTPUT;
+    // the GELU epilogue exists in the direct-to-LDS kernel only
+    if (in % 32 != 0 || out % 8 != 0 || !aligned16(x) || !aligned16(w) || !aligned16(u) || !aligned16(y))
+        return BR_ERR_TODO;
+    GemmArgs g;
+    g.a = x; g.b = w; g.c = u; g.c2 = y; g.bias = bias;
+    g.m = rows; g.n = out; g.k = in;
+    g.lda = in; g.ldb = in; g.ldc = out;
+    g.sa = g.sb = g.sc = 0;
+    g.alpha = 1.0f;
+    g.accumulate = 0;
+    g.tiles_m = g.tiles_n = 0;  // set by the launcher for the tile it picks
+    g.vec_a = g.vec_b = 1;
+    gemm16::Problem p;
+    p.a_f32 = p.b_f32 = false;
+    p.a_kstr = p.b_kstr = false;
+    p.c_dtype = dtype;
+    p.guarded = false;
+    hipStream_t st = as_stream(stream);
+    if (dtype == BR_F16) return gemm16_launch_f16(g, p, 1, st);
+    return gemm16_launch_bf16(g, p, 1, st);
+}
+
 // ---- fp32 operands staged as 16-bit copies ----------------------------------
 namespace {
 

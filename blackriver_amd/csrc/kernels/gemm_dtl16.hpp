@@ -141,7 +141,8 @@ struct DtlTile {
     }
 };
 
-template <int CT, int BM, int BN, int WM, int WN, int KT, int STAGES, bool A_KSTR, bool B_KSTR, typename TC>
+template <int CT, int BM, int BN, int WM, int WN, int KT, int STAGES, bool A_KSTR, bool B_KSTR, typename TC,
+          bool GELU = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(GemmArgs g) {
     constexpr int WAVES = (BM / WM) * (BN / WN);
     constexpr int FM = WM / 32, FN = WN / 32, KS = KT / 16;
@@ -284,6 +285,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     // acc[i][j][v] is C[row, col] with
     //   row = wm*WM + i*32 + (v/4)*8 + (lane/32)*4 + v%4,  col = wn*WN + j*32 + lane%32
     TC* c_base = static_cast<TC*>(g.c) + batch * g.sc;
+    TC* c2_base = GELU ? static_cast<TC*>(g.c2) + batch * g.sc : nullptr;
 #pragma unroll
     for (int j = 0; j < FN; j++) {
         const long long col = col0 + wn * WN + j * 32 + (lane & 31);
@@ -299,6 +301,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                     float o = g.alpha * acc[i][j][v] + bias;
                     if (g.accumulate) o += c_load<TC>(p);
                     c_store<TC>(p, o);
+                    // the activation is taken of the fp32 value, not of its rounded copy
+                    if (GELU) c_store<TC>(c2_base + row * g.ldc + col, gelu_one(o));
                 }
             }
         }
@@ -316,6 +320,16 @@ int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t
     const unsigned grid = (unsigned)blocks;
     using F16 = __half;
     using BF16 = __hip_bfloat16;
+    if (g.c2) {
+        // GELU epilogue: built for the linear layer's layout only (both operands k-contiguous, 16-bit outputs)
+        if (p.a_kstr || p.b_kstr || p.c_dtype == BR_F32) return BR_ERR_TODO;
+        if (CT == BR_GEMM_F16)
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, false, false, F16, true><<<grid, THREADS, 0, st>>>(g);
+        else
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, false, false, BF16, true><<<grid, THREADS, 0, st>>>(g);
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
+    }
 #define BR_DTL_CASE(AK, BK_)                                                                           \
     if (p.a_kstr == AK && p.b_kstr == BK_) {                                                            \
         if (p.c_dtype == BR_F32)                                                                        \
@@ -387,6 +401,7 @@ int launch_dtl(const GemmArgs& g, const Problem& p, long long batch, hipStream_t
 template <int CT>
 int launch_any(const GemmArgs& g, const Problem& p, long long batch, hipStream_t st) {
     if (dtl_applies(g, p)) return launch_dtl<CT>(g, p, batch, st);
+    if (g.c2) return BR_ERR_TODO;  // only the direct-to-LDS kernel has the GELU epilogue
     return launch<CT>(g, p, batch, st);
 }
 

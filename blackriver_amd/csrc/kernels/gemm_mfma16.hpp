@@ -64,6 +64,9 @@ struct GemmArgs {
     int accumulate;
     int tiles_m, tiles_n;
     int vec_a, vec_b;  // 128-bit global loads allowed for this operand
+    // second output of the direct-to-LDS kernel's GELU epilogue: gelu of what
+    // goes to c, same layout and type as c (null = plain epilogue)
+    void* c2 = nullptr;
 };
 
 template <int CT>

@@ -112,13 +112,15 @@ int br_hip_gelu_bwd(const void* dy, const void* x, void* dx, int dtype, int64_t 
  * cuda_tensor.cpp:180-190 fused with kernels::gelu_forward.  bias is fp32. */
 int br_hip_bias_gelu_fwd(const void* x, const float* bias, void* y, int dtype, int64_t rows,
                          int64_t cols, br_stream_t stream);
-/* dx = dy * gelu'(x + bias); when dbias != NULL also dbias[col] = sum_rows dx
- * (the cudnnReduceTensor of cuda_tensor.cpp:738-760).  workspace must hold
- * br_hip_bias_gelu_bwd_workspace(rows, cols) bytes when dbias != NULL. */
+/* dx = dy * gelu'(x + bias) (bias may be NULL: x already holds it); when
+ * dbias != NULL also dbias[col] = dbias_scale * sum_rows dx (the
+ * cudnnReduceTensor of cuda_tensor.cpp:738-760; the sum is over dx as stored).
+ * workspace must hold br_hip_bias_gelu_bwd_workspace(rows, cols) bytes when
+ * dbias != NULL. */
 size_t br_hip_bias_gelu_bwd_workspace(int64_t rows, int64_t cols);
 int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void* dx,
-                         float* dbias, int dtype, int64_t rows, int64_t cols, void* workspace,
-                         size_t workspace_bytes, br_stream_t stream);
+                         float* dbias, int dtype, int64_t rows, int64_t cols, float dbias_scale,
+                         void* workspace, size_t workspace_bytes, br_stream_t stream);
 
 /* kernels::launch_transform_0213<float>, kernels/transform_kernels.cu:56-65
  * (declared kernels/kernels.h:35), called at cuda_tensor.cpp:257-275: [s0,s1,s2,s3] -> [s0,s2,s1,s3].
@@ -328,6 +330,18 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
                        int accumulate, void* c, int c_dtype, int64_t ldc, int64_t stride_c,
                        const float* bias, int64_t batch, int compute,
                        void* workspace, size_t workspace_bytes, br_stream_t stream);
+
+/* op_linear followed by op_gelu (cuda_tensor.cpp:146-193 and :400-412; the pair
+ * of bloomz-7b/train.words:188-189) in one product whose epilogue writes both
+ * tensors the backward pass needs, in the products' own 16-bit type:
+ *   u[r, o] = sum_i x[r, i] * w[o, i] + bias[o]      y[r, o] = gelu(u[r, o])
+ * x [rows, in], w [out, in], u and y [rows, out] are dense, all of `dtype`
+ * (BR_F16 or BR_BF16); bias fp32 (may be NULL).  The activation is evaluated on
+ * the fp32 sum, before u is rounded.  BR_ERR_TODO when the shape or alignment
+ * rules out the direct-to-LDS kernel (in % 32, 16-byte aligned rows): the
+ * caller then runs the two operators. */
+int br_hip_linear_gelu(const void* x, const void* w, const float* bias, void* u, void* y, int dtype,
+                       int64_t rows, int64_t out, int64_t in, br_stream_t stream);
 
 /* ---- fused attention --------------------------------------------------- */
 /* The operator chain of bloomz-7b/train.words:154-166 in one kernel:

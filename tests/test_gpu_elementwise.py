@@ -48,7 +48,7 @@ def test_bias_gelu_f16_headline_shape():
     dbias = empty(cols)
     call("br_hip_bias_gelu_fwd", ptr(dx_), ptr(db_), ptr(y), F16, rows, cols, stream())
     ws = workspace(hip.load().br_hip_bias_gelu_bwd_workspace(rows, cols))
-    call("br_hip_bias_gelu_bwd", ptr(dy_), ptr(dx_), ptr(db_), ptr(g), ptr(dbias), F16, rows, cols, ptr(ws),
+    call("br_hip_bias_gelu_bwd", ptr(dy_), ptr(dx_), ptr(db_), ptr(g), ptr(dbias), F16, rows, cols, 1.0, ptr(ws),
          ws.numel(), stream())
     x32, dy32 = x.astype(np.float32), dy.astype(np.float32)
     assert_close_f16(host(y), orc.bias_gelu_fwd(x32, bias), RTOL, "bias gelu fwd (fp16 storage)")
@@ -70,7 +70,7 @@ def test_bias_gelu_small_and_unaligned(rows, cols, dtype):
     y, g, dbias = empty((rows, cols), t_t), empty((rows, cols), t_t), empty(cols)
     call("br_hip_bias_gelu_fwd", ptr(dx_), ptr(db_), ptr(y), code, rows, cols, stream())
     ws = workspace(hip.load().br_hip_bias_gelu_bwd_workspace(rows, cols))
-    call("br_hip_bias_gelu_bwd", ptr(dy_), ptr(dx_), ptr(db_), ptr(g), ptr(dbias), code, rows, cols, ptr(ws),
+    call("br_hip_bias_gelu_bwd", ptr(dy_), ptr(dx_), ptr(db_), ptr(g), ptr(dbias), code, rows, cols, 1.0, ptr(ws),
          ws.numel(), stream())
     y_ref = orc.bias_gelu_fwd(x.astype(np.float32), bias)
     g_ref, dbias_ref = orc.bias_gelu_bwd(dy.astype(np.float32), x.astype(np.float32), bias)

@@ -259,3 +259,31 @@ def test_gemm_rejects_bad_arguments():
     assert lib.br_hip_gemm(0, 1, 8, 8, 8, 1.0, ptr(t), F32, 8, 0, ptr(t), F32, 8, 0, 0, None, F32, 8, 0, None, 1,
                            hip.GEMM_F16, stream()) == -3
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype", [F16, BF16])
+@pytest.mark.parametrize("rows,out,inn", [(512, 1024, 256), (200, 520, 96), (2048, 4096, 1024)])
+def test_linear_gelu_epilogue_writes_both_tensors(dtype, rows, out, inn):
+    """br_hip_linear_gelu: u = x.W^T + bias and y = gelu(u) from one product.
+    u against the fp64 product of the stored operands, y against the oracle's
+    GELU of that fp64 u (the kernel takes the activation of the fp32 sum, so y
+    does not inherit u's storage rounding); 2e-2 for 16-bit operands, plus the
+    output's own rounding."""
+    import oracle as orc
+    print("case dtype=%d rows=%d out=%d in=%d" % (dtype, rows, out, inn), flush=True)
+    rng = np.random.default_rng(rows + out)
+    x = to_dev(rng.standard_normal((rows, inn)), dtype)
+    w = to_dev(rng.standard_normal((out, inn)) / np.sqrt(inn) * 1.5, dtype)
+    bias = (0.1 * rng.standard_normal(out)).astype(np.float32)
+    u = torch.full((rows, out), float("nan"), dtype=TORCH_T[dtype], device="cuda")
+    y = torch.full((rows, out), float("nan"), dtype=TORCH_T[dtype], device="cuda")
+    call("br_hip_linear_gelu", ptr(x), ptr(w), ptr(dev(bias)), ptr(u), ptr(y), dtype, rows, out, inn, stream())
+    ref_u = to_host64(x) @ to_host64(w).T + bias.astype(np.float64)
+    ref_y = orc.gelu_fwd(ref_u.astype(np.float32)).astype(np.float64)
+    tol = 2e-2 if dtype == F16 else 3e-2
+    assert_close(to_host64(u), ref_u, tol, "pre-activation")
+    assert_close(to_host64(y), ref_y, tol, "gelu")
+    # shapes the direct-to-LDS kernel does not take are declined, nothing is written
+    assert hip.load().br_hip_linear_gelu(ptr(x), ptr(w), None, ptr(u), ptr(y), dtype, rows, out, inn - 8, stream()) == -1
+    assert hip.load().br_hip_linear_gelu(ptr(x), ptr(w), None, ptr(u), ptr(u), dtype, rows, out, inn, stream()) == -3
+    torch.cuda.synchronize()
