@@ -201,11 +201,16 @@ def roofline_leg(hip, timer, torch, full):
             "traffic": ROOFLINE_TRAFFIC_BYTES}
     # what a bare MFMA loop (no memory traffic) reaches on this box with operands of zeros and of random values
     scratch = torch.empty(1 << 17, device="cuda")
+    probe = ctypes.CDLL(os.path.join(ROOT, "blackriver_amd", "lib", "libbr_probe.so"))
+    probe.br_probe_mfma_f16.restype = ctypes.c_int
+    probe.br_probe_mfma_f16.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64,
+                                        ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
     loop = {}
     for name, rnd in (("zeros", 0), ("random", 1)):
         tf = ctypes.c_double()
-        hip.call("br_hip_probe_mfma_f16", rnd, 8000, ctypes.c_void_p(scratch.data_ptr()), scratch.numel(),
-                 ctypes.byref(tf), timer.stream)
+        rc = probe.br_probe_mfma_f16(rnd, 8000, ctypes.c_void_p(scratch.data_ptr()), scratch.numel(), ctypes.byref(tf),
+                                     timer.stream)
+        assert rc == 0, "MFMA calibration loop failed with %d" % rc
         loop[name] = round(tf.value, 1)
     roof["mfma_loop_tflops"] = loop
     roof["frac_of_random_operand_loop"] = roof["achieved"] / loop["random"]

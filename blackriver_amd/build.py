@@ -3,6 +3,18 @@
   libbr_hip.so       HIP kernels + C ABI (hipcc, gfx950 only)
   libblackriver.so   C++ host runtime: operator API, tensors, word VM
                      (g++, links libbr_hip.so; never includes a HIP header)
+  libbr_probe.so     the bare-MFMA calibration loop bench.py reports beside
+                     the GEMM figures (measurement aid; the product never
+                     loads it)
+
+``python -m blackriver_amd.build --sanitize`` builds, into lib/sanitize/, the
+host runtime and the CPU oracle with AddressSanitizer + UBSan (host code only;
+the kernel library is linked as built) for running the CPU test suite under
+the sanitizers:
+    LD_PRELOAD="$(gcc -print-file-name=libasan.so) $(gcc -print-file-name=libstdc++.so)" \
+        BR_SANITIZE=1 ASAN_OPTIONS=detect_leaks=0 python -m pytest tests -m "not gpu"
+(libstdc++ is preloaded with libasan so that the interceptor of C++ throws finds
+the real function inside an interpreter that is not linked against it.)
 
 Run as ``python -m blackriver_amd.build``.  hipcc cross-compiles for gfx950
 without a GPU, so this works on a CPU-only machine.
@@ -22,6 +34,10 @@ HOST_DIR = os.path.join(PKG, "csrc", "host")
 LIB_DIR = os.path.join(PKG, "lib")
 OBJ_DIR = os.path.join(PKG, "build")
 
+BENCH_DIR = os.path.join(PKG, "csrc", "bench")
+PROBE_LIB = os.path.join(LIB_DIR, "libbr_probe.so")
+SAN_DIR = os.path.join(LIB_DIR, "sanitize")
+SAN_FLAGS = ["-fsanitize=address,undefined", "-fno-omit-frame-pointer", "-g", "-O1"]
 HIP_LIB = os.path.join(LIB_DIR, "libbr_hip.so")
 HOST_LIB = os.path.join(LIB_DIR, "libblackriver.so")
 
@@ -103,12 +119,43 @@ def build_host(verbose=True, force=True):
     return HOST_LIB
 
 
+def build_probe(verbose=True):
+    """The calibration loop of bench.py: its own small library."""
+    src = os.path.join(BENCH_DIR, "probe.hip")
+    _run(["hipcc"] + HIPCC_FLAGS + ["-shared", "-o", PROBE_LIB, src])
+    if verbose:
+        print("built", PROBE_LIB)
+    return PROBE_LIB
+
+
+def build_sanitized(verbose=True):
+    """Host runtime and CPU oracle with ASan + UBSan (host compilers only)."""
+    os.makedirs(SAN_DIR, exist_ok=True)
+    srcs = _sources(HOST_DIR, ".cpp")
+    host = os.path.join(SAN_DIR, "libblackriver.so")
+    _run(["g++"] + CXX_FLAGS + SAN_FLAGS + ["-shared", "-o", host] + srcs +
+         ["-L" + LIB_DIR, "-lbr_hip", "-Wl,-rpath,$ORIGIN/.."])
+    oracle = os.path.join(SAN_DIR, "libbr_oracle.so")
+    _run(["gcc", "-fopenmp", "-march=x86-64-v3", "-fPIC", "-std=c11", "-Wall", "-Wextra"] + SAN_FLAGS +
+         ["-shared", "-o", oracle, os.path.join(ROOT, "oracle", "br_oracle.c"), "-lm"])
+    if verbose:
+        print("built", host)
+        print("built", oracle)
+    return host, oracle
+
+
 def build_all(verbose=True, force=True):
     build_kernels(verbose, force)
     build_host(verbose, force)
+    build_probe(verbose)
 
 
 if __name__ == "__main__":
     # `--incremental` recompiles only sources that changed since the last build
-    build_all(force="--incremental" not in sys.argv)
+    if "--sanitize" in sys.argv:
+        if not os.path.exists(HIP_LIB):
+            build_kernels()
+        build_sanitized()
+    else:
+        build_all(force="--incremental" not in sys.argv)
     sys.exit(0)

@@ -3,11 +3,12 @@
 // MI355X the two differ by a third -- the clock follows the switching activity
 // of the data -- so a GEMM on real data has to be read against the second
 // figure as well as against the nominal peak.
-#include "common.hpp"
-
+//
+// Built into libbr_probe.so, which only bench.py loads: a measuring aid, not
+// part of the kernel library or of its C ABI.
+#include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
-
-using namespace brk;
+#include <stdint.h>
 
 namespace {
 
@@ -58,11 +59,19 @@ __global__ __launch_bounds__(512) void mfma_loop_kernel(float* out, int passes) 
 
 }  // namespace
 
-extern "C" int br_hip_probe_mfma_f16(int random_operands, int passes, float* scratch, int64_t scratch_floats,
-                                     double* tflops, br_stream_t stream) {
+#define BR_HIP_TRY(expr)                                \
+    do {                                                \
+        hipError_t br_err_ = (expr);                    \
+        if (br_err_ != hipSuccess) return (int)br_err_; \
+    } while (0)
+
+// Returns 0, a hipError_t, or -4 for bad arguments.  scratch: at least 131072
+// floats of device memory; *tflops receives the rate of the timed launch.
+extern "C" int br_probe_mfma_f16(int random_operands, int passes, float* scratch, int64_t scratch_floats,
+                                 double* tflops, void* stream) {
     const int blocks = 256;
-    if (passes < 1 || !scratch || scratch_floats < (int64_t)blocks * 512 || !tflops) return BR_ERR_ATTR;
-    hipStream_t st = as_stream(stream);
+    if (passes < 1 || !scratch || scratch_floats < (int64_t)blocks * 512 || !tflops) return -4;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     hipEvent_t e0, e1;
     BR_HIP_TRY(hipEventCreate(&e0));
     BR_HIP_TRY(hipEventCreate(&e1));
@@ -79,7 +88,7 @@ extern "C" int br_hip_probe_mfma_f16(int random_operands, int passes, float* scr
     BR_HIP_TRY(hipEventElapsedTime(&ms, e0, e1));
     BR_HIP_TRY(hipEventDestroy(e0));
     BR_HIP_TRY(hipEventDestroy(e1));
-    BR_HIP_LAUNCH_CHECK();
+    BR_HIP_TRY(hipGetLastError());
     *tflops = (double)blocks * 8.0 * passes * 64.0 * 2.0 * 32 * 32 * 16 / ((double)ms * 1e-3) / 1e12;
-    return BR_OK;
+    return 0;
 }

@@ -265,6 +265,7 @@ __device__ __forceinline__ void c_store<__half>(__half* p, float v) { *p = __flo
 template <>
 __device__ __forceinline__ void c_store<__hip_bfloat16>(__hip_bfloat16* p, float v) { *p = __float2bfloat16(v); }
 
+
 // Workgroup id -> (batch, tile_m, tile_n).
 __device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch, int& tm, int& tn) {
     const long long nb = gridDim.x;

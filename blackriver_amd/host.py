@@ -11,7 +11,10 @@ import os
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libblackriver.so")
+# BR_SANITIZE=1 selects the ASan + UBSan build of the host runtime
+# (`python -m blackriver_amd.build --sanitize`; the interpreter then needs
+# libasan preloaded)
+LIB_PATH = os.path.join(_PKG, "lib", "sanitize" if os.environ.get("BR_SANITIZE") == "1" else "", "libblackriver.so")
 WORDS_DIR = os.path.join(_PKG, "words")
 
 _vp = ctypes.c_void_p

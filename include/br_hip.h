@@ -399,16 +399,6 @@ int br_hip_adamw(void* param, int param_dtype, float* master, const float* grad,
                  int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
                  int64_t step, br_stream_t stream);
 
-/* ---- calibration ------------------------------------------------------- */
-/* Rate of a bare v_mfma_f32_32x32x16_f16 loop without any memory traffic, with
- * operands of zeros (random_operands == 0) or of random values: on MI355X the
- * clock follows the switching activity of the data, so the second figure, not
- * the nominal peak, is what a GEMM on real data can approach.  scratch: at
- * least 131072 floats of device memory.  Measurement only; nothing in the
- * reference corresponds to it. */
-int br_hip_probe_mfma_f16(int random_operands, int passes, float* scratch, int64_t scratch_floats,
-                          double* tflops, br_stream_t stream);
-
 /* ---- data preparation (bit-exact integer / gather work) ---------------- */
 /* The embedding row gather of blackriver/train_bloom.cpp:50-56. */
 int br_hip_embedding_gather(const void* table, const int32_t* ids, void* out, int elem_bytes,

@@ -17,6 +17,8 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libbr_oracle.so")
+if os.environ.get("BR_SANITIZE") == "1":   # the ASan + UBSan build made by `python -m blackriver_amd.build --sanitize`
+    _LIB_PATH = os.path.join(os.path.dirname(_HERE), "blackriver_amd", "lib", "sanitize", "libbr_oracle.so")
 _lib = None
 
 _f32p = ctypes.POINTER(ctypes.c_float)

@@ -195,15 +195,6 @@ def test_normal_fill_is_a_function_of_seed_and_index():
     assert np.all(np.isfinite(va))
 
 
-def test_mfma_probe_reports_a_rate():
-    scratch = empty(1 << 17)
-    for rnd in (0, 1):
-        tf = ctypes.c_double()
-        call("br_hip_probe_mfma_f16", rnd, 200, ptr(scratch), scratch.numel(), ctypes.byref(tf), stream())
-        assert 100.0 < tf.value < 5000.0
-    assert hip.load().br_hip_probe_mfma_f16(0, 200, ptr(scratch), 10, ctypes.byref(tf), stream()) == -4
-
-
 def test_fill_and_cast_roundtrip():
     n = 100003
     t = empty(n)
