@@ -483,6 +483,12 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
     const float* x = static_cast<const float*>(mem_);
     float* dx = static_cast<float*>(x_g->data());
     float* logits = static_cast<float*>(all_logits->data());
+    // lm_head_g is accumulated into, as the reference does; a driver that would
+    // zero it right before (ComputingContext::loss_head_overwrite) gets the
+    // first chunk written instead of added, which saves clearing and re-reading
+    // a [vocab, hidden] tensor
+    bool overwrite = ComputingContext::loss_head_overwrite && lm_head_g->is_cuda();
+    if (overwrite && count == 0) BR_OP(br_hip_fill(d_wg, BR_F32, 0.f, vocab * hidden, stream()));
     for (int64_t r0 = 0; r0 < n && count > 0; r0 += cap) {
         const int64_t rows = std::min(cap, n - r0);
         bool any = false;
@@ -521,8 +527,11 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
         BR_OP(product(0, 0, rows, hidden, vocab, alpha * grad_lift, dl.ptr, dl.dtype, vocab, 0, lm_head->data(), code(lm_head),
                       hidden, 0, 0, dx + r0 * hidden, BR_F32, hidden, 0, nullptr, 1, compute));
         BR_OP(product(1, 0, vocab, hidden, rows, alpha, dl.ptr, dl.dtype, vocab, 0, x + r0 * hidden, BR_F32, hidden,
-                      0, 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
+                      0, overwrite ? 0 : 1, d_wg, BR_F32, hidden, 0, nullptr, 1, compute));
+        overwrite = false;
     }
+    // overwrite mode with no chunk carrying a label at all: the gradient is zero
+    if (overwrite && count > 0) BR_OP(br_hip_fill(d_wg, BR_F32, 0.f, vocab * hidden, stream()));
 
     // sum of log p(label) in fp64 on the host, as the reference accumulates it
     std::vector<float> logp(n, 0.f);

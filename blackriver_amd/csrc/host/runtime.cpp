@@ -56,6 +56,7 @@ float ComputingContext::last_loss = 0.0f;
 bool ComputingContext::echo_loss = true;
 float ComputingContext::grad_lift = 1.0f;
 bool ComputingContext::grad_lift_auto = false;
+bool ComputingContext::loss_head_overwrite = false;
 void* ComputingContext::scratch_ptr_ = nullptr;
 size_t ComputingContext::scratch_size_ = 0;
 void* ComputingContext::staging_ptr_[2] = {nullptr, nullptr};

@@ -41,6 +41,9 @@ struct ComputingContext {
     // S = 16 * 2^ceil(log2(count)) itself when the products run in 16 bit.
     static float grad_lift;
     static bool grad_lift_auto;
+    // op_loss_backward overwrites a device-resident lm_head_g instead of adding
+    // to it (set for the duration of the word op.loss_backward_set)
+    static bool loss_head_overwrite;
 
     static void boot(int dev);  // 128 MiB of scratch like context.cpp:31
     static void shutdown();

@@ -224,6 +224,15 @@ BR_WORD(Gelu, Tensors<2> a(stack); a[0]->op_gelu(a[0], a[1]);)
 BR_WORD(LastLogits, Tensors<4> a(stack); a[0]->op_last_logits(a[0], a[1], a[2], a[3]);)
 // ( x ids mask lm_head workspace x_g lm_head_g -- )
 BR_WORD(LossBackward, Tensors<7> a(stack); a[0]->op_loss_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6]);)
+// ( x ids mask lm_head workspace x_g lm_head_g -- )  the same with lm_head_g
+// overwritten: `'lm_head_g' @ op.zero` followed by op.loss_backward without
+// the clearing pass and the re-read of a [vocab, hidden] tensor (extension)
+BR_WORD(LossBackwardSet,
+    Tensors<7> a(stack);
+    ComputingContext::loss_head_overwrite = true;
+    a[0]->op_loss_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6]);
+    ComputingContext::loss_head_overwrite = false;
+)
 // ( dy scale bias var y dscale dbias din eps -- )
 BR_WORD(LayernormBackward,
     const float eps = (float)stack.pop_number();
@@ -465,6 +474,7 @@ void load_nn_words(Enviroment& env) {
         {"op.gelu", Gelu::creator},
         {"op.last_logits", LastLogits::creator},
         {"op.loss_backward", LossBackward::creator},
+        {"op.loss_backward_set", LossBackwardSet::creator},
         {"op.layernorm_backward", LayernormBackward::creator},
         {"op.linear_backward", LinearBackward::creator},
         {"op.gelu_backward", GeluBackward::creator},

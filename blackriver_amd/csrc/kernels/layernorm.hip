@@ -112,19 +112,29 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic(const float* x, const f
 }
 
 // --------------------------------------------------------------- backward
-template <int VPT>
-__global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* dy, const float* __restrict__ y,
-                                                       const float* __restrict__ gamma,
-                                                       const float* __restrict__ beta,
-                                                       const float* __restrict__ var, float* dx,
-                                                       float* __restrict__ part_dgamma,
-                                                       float* __restrict__ part_dbeta, int64_t rows, int cols4,
-                                                       float eps, float inv_cols, const float* residual) {
-    __shared__ float lds[2][2 * kWaves];
+// A workgroup is GROUPS row walkers of 256 threads each: walker w of workgroup
+// b takes rows (b*GROUPS + w), + gridDim.x*GROUPS, ...; each keeps gamma, beta,
+// 1/gamma and its running dgamma / dbeta in registers and has the next row's
+// loads in flight while it works on the current one.  At the end the walkers'
+// running sums are added in LDS (walker order) and the workgroup writes ONE
+// partial row pair, so the finalize pass reads gridDim.x partials.
+constexpr int kWalker = kBlock;  // threads per row walker
+template <int VPT, int GROUPS>
+__global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy, const float* __restrict__ y,
+                                                                 const float* __restrict__ gamma,
+                                                                 const float* __restrict__ beta,
+                                                                 const float* __restrict__ var, float* dx,
+                                                                 float* __restrict__ part_dgamma,
+                                                                 float* __restrict__ part_dbeta, int64_t rows,
+                                                                 int cols4, float eps, float inv_cols,
+                                                                 const float* residual) {
+    __shared__ float lds[2][GROUPS][2 * kWaves];
+    const int walker = threadIdx.x / kWalker, tid = threadIdx.x % kWalker;
+    const int lane = tid & 63, wave = tid >> 6;
     float4 g[VPT], ginv[VPT], b[VPT], acc_g[VPT], acc_b[VPT];
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
-        const int idx = threadIdx.x + i * kBlock;
+        const int idx = tid + i * kWalker;
         const bool ok = idx < cols4;
         g[i] = ok ? reinterpret_cast<const float4*>(gamma)[idx] : make_float4(1.f, 1.f, 1.f, 1.f);
         b[i] = ok ? reinterpret_cast<const float4*>(beta)[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -133,27 +143,31 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* dy, const flo
         acc_g[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         acc_b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    // The next row's dy / y are requested before the current row is worked on,
-    // so two rows per workgroup are in flight.
     float4 d[VPT], xh[VPT], nd[VPT], nxh[VPT];
+    // rows past the end read as dy = 0, y = beta: they add nothing to any sum
     auto request = [&](float4 (&rd)[VPT], float4 (&ry)[VPT], int64_t row) {
         const float4* dyr = reinterpret_cast<const float4*>(dy) + row * cols4;
         const float4* yr = reinterpret_cast<const float4*>(y) + row * cols4;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
-            const int idx = threadIdx.x + i * kBlock;
-            const bool ok = idx < cols4;
+            const int idx = tid + i * kWalker;
+            const bool ok = idx < cols4 && row < rows;
             rd[i] = ok ? dyr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
             ry[i] = ok ? yr[idx] : b[i];
         }
     };
-    if (blockIdx.x < rows) request(d, xh, blockIdx.x);
+    const int64_t stride = (int64_t)gridDim.x * GROUPS;
+    const int64_t first = (int64_t)blockIdx.x * GROUPS + walker;
+    // every walker of a workgroup makes the same number of trips (they share barriers)
+    const int64_t trips = (rows - (int64_t)blockIdx.x * GROUPS + stride - 1) / stride;
+    request(d, xh, first);
     int flip = 0;
-    for (int64_t row = blockIdx.x; row < rows; row += gridDim.x, flip ^= 1) {
-        const int64_t next = row + gridDim.x;
-        if (next < rows) request(nd, nxh, next);
+    for (int64_t trip = 0; trip < trips; trip++, flip ^= 1) {
+        const int64_t row = first + trip * stride;
+        const bool live = row < rows;
+        request(nd, nxh, row + stride);
         // stored var already holds eps; the backward adds eps once more
-        const float rstd = 1.0f / sqrtf(var[row] + eps);
+        const float rstd = live ? 1.0f / sqrtf(var[row] + eps) : 0.f;
         // optional residual gradient added to dx (dx may be the same buffer):
         // requested here so that its latency hides behind the row reduction
         float4 res[VPT];
@@ -161,8 +175,8 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* dy, const flo
             const float4* rr = reinterpret_cast<const float4*>(residual) + row * cols4;
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
-                const int idx = threadIdx.x + i * kBlock;
-                res[i] = idx < cols4 ? rr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+                const int idx = tid + i * kWalker;
+                res[i] = (idx < cols4 && live) ? rr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }
         float s[2] = {0.f, 0.f};
@@ -180,13 +194,26 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* dy, const flo
             s[0] += (d[i].x + d[i].y) + (d[i].z + d[i].w);
             s[1] += (d[i].x * xh[i].x + d[i].y * xh[i].y) + (d[i].z * xh[i].z + d[i].w * xh[i].w);
         }
-        block_sum<2>(s, lds[flip]);
+        // the walker's two row sums: wave butterflies, then its four waves through LDS
+        s[0] = wave_sum(s[0]);
+        s[1] = wave_sum(s[1]);
+        if (lane == 0) {
+            lds[flip][walker][wave] = s[0];
+            lds[flip][walker][kWaves + wave] = s[1];
+        }
+        __syncthreads();
+        s[0] = s[1] = 0.f;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) {
+            s[0] += lds[flip][walker][w];
+            s[1] += lds[flip][walker][kWaves + w];
+        }
         const float m1 = s[0] * inv_cols, m2 = s[1] * inv_cols;
         float4* dxr = reinterpret_cast<float4*>(dx) + row * cols4;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
-            const int idx = threadIdx.x + i * kBlock;
-            if (idx < cols4) {
+            const int idx = tid + i * kWalker;
+            if (idx < cols4 && live) {
                 float4 o;
                 o.x = (d[i].x - m1 - xh[i].x * m2) * rstd;
                 o.y = (d[i].y - m1 - xh[i].y * m2) * rstd;
@@ -206,14 +233,39 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_regs(const float* dy, const flo
             xh[i] = nxh[i];
         }
     }
-    float4* pg = reinterpret_cast<float4*>(part_dgamma) + (int64_t)blockIdx.x * cols4;
-    float4* pb = reinterpret_cast<float4*>(part_dbeta) + (int64_t)blockIdx.x * cols4;
+    // walkers 1.. hand their running sums to walker 0 through LDS, in walker order
+    if (GROUPS > 1) {
+        __shared__ float4 hand[2][VPT][kWalker];
+        for (int w = 1; w < GROUPS; w++) {
+            __syncthreads();
+            if (walker == w) {
 #pragma unroll
-    for (int i = 0; i < VPT; i++) {
-        const int idx = threadIdx.x + i * kBlock;
-        if (idx < cols4) {
-            pg[idx] = acc_g[i];
-            pb[idx] = acc_b[i];
+                for (int i = 0; i < VPT; i++) {
+                    hand[0][i][tid] = acc_g[i];
+                    hand[1][i][tid] = acc_b[i];
+                }
+            }
+            __syncthreads();
+            if (walker == 0) {
+#pragma unroll
+                for (int i = 0; i < VPT; i++) {
+                    const float4 a = hand[0][i][tid], c = hand[1][i][tid];
+                    acc_g[i].x += a.x; acc_g[i].y += a.y; acc_g[i].z += a.z; acc_g[i].w += a.w;
+                    acc_b[i].x += c.x; acc_b[i].y += c.y; acc_b[i].z += c.z; acc_b[i].w += c.w;
+                }
+            }
+        }
+    }
+    if (walker == 0) {
+        float4* pg = reinterpret_cast<float4*>(part_dgamma) + (int64_t)blockIdx.x * cols4;
+        float4* pb = reinterpret_cast<float4*>(part_dbeta) + (int64_t)blockIdx.x * cols4;
+#pragma unroll
+        for (int i = 0; i < VPT; i++) {
+            const int idx = tid + i * kWalker;
+            if (idx < cols4) {
+                pg[idx] = acc_g[i];
+                pb[idx] = acc_b[i];
+            }
         }
     }
 }
@@ -330,11 +382,14 @@ __global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restr
     }
 }
 
+// Persistent workgroups of the register path: one per CU on a 256-CU part, two
+// row walkers each (512 rows in flight chip-wide, 256 partial row pairs).
+constexpr int kBwdWalkers = 2;
 int bwd_parts(int64_t rows) {
-    // persistent workgroups: two per CU on a 256-CU part, never more than rows
     static const char* e = getenv("BR_LN_PARTS");
-    int64_t p = e ? atoi(e) : 512;
-    if (p > rows) p = rows;
+    int64_t p = e ? atoi(e) : 256;
+    const int64_t most = (rows + kBwdWalkers - 1) / kBwdWalkers;
+    if (p > most) p = most;
     return (int)(p < 1 ? 1 : p);
 }
 
@@ -464,18 +519,15 @@ static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamm
         const int cols4 = (int)(cols / 4);
         const float inv = 1.0f / (float)cols;
         const int vpt = (cols4 + kBlock - 1) / kBlock;
-        if (vpt <= 1)
-            ln_bwd_regs<1><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
-                                                     residual);
-        else if (vpt <= 2)
-            ln_bwd_regs<2><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
-                                                     residual);
-        else if (vpt <= 4)
-            ln_bwd_regs<4><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
-                                                     residual);
-        else
-            ln_bwd_regs<8><<<parts, kBlock, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, inv,
-                                                     residual);
+        constexpr int G = kBwdWalkers;
+#define BR_LN_BWD(V)                                                                                              \
+    ln_bwd_regs<V, G><<<parts, kWalker * G, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, \
+                                                     inv, residual)
+        if (vpt <= 1) BR_LN_BWD(1);
+        else if (vpt <= 2) BR_LN_BWD(2);
+        else if (vpt <= 4) BR_LN_BWD(4);
+        else BR_LN_BWD(8);
+#undef BR_LN_BWD
         BR_HIP_LAUNCH_CHECK();
         if (aligned16(dgamma) && aligned16(dbeta))
             ln_bwd_finalize_x4<<<(unsigned)((cols4 + 15) / 16), 1024, 0, st>>>(

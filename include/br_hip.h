@@ -192,7 +192,7 @@ int br_hip_layernorm_bwd(const float* dy, const float* y, const float* gamma,
  * life of the process); the call makes no hipMalloc / hipFree and uses the
  * same kernels as br_hip_layernorm_bwd, so results are identical bit for bit.
  * Returns BR_ERR_SCRATCH when br_hip_layernorm_bwd_workspace(rows, cols)
- * exceeds the limit (e.g. cols > 4096 at 512 or more rows).  All calls on one
+ * exceeds the limit (e.g. cols > 8192 at 512 or more rows).  All calls on one
  * GPU share the buffer: calls that overlap in time on one GPU (two streams)
  * race; calls on one stream, or ordered by events, are safe. */
 size_t br_hip_layernorm_bwd_static_limit(void);

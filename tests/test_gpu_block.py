@@ -159,6 +159,12 @@ def test_loss_head_against_oracle(runtime, mode):
     loss_ref, xg_ref, wg_ref, _ = orc.loss_backward(x, ids, mask, lm, lm_head_g=g0)
     assert_close(env.read("xa"), xg_ref, tol, "x_g")
     assert_close(env.read("lm_head.weight_g"), wg_ref, tol, "lm_head_g (accumulated)")
+    # the overwriting form: whatever the gradient tensor held is gone, the result is the sum alone
+    env.write("lm_head.weight_g", g0 * 7)
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xb' @ 'lm_head.weight_g' @ "
+                "op.loss_backward_set op.sync")
+    assert_close(env.read("lm_head.weight_g"), wg_ref - g0, tol, "lm_head_g (overwritten)")
+    assert np.array_equal(env.read("xb"), env.read("xa"))
     # a second call with a CPU gradient tensor, as the reference keeps it
     env.execute("%d %d 2 'cpu' 'float' op.create 'lm_g_cpu' !  'lm_g_cpu' @ op.zero" % (vocab, hidden))
     env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xb' @ 'lm_g_cpu' @ op.loss_backward")

@@ -49,8 +49,8 @@ def both_entries(rows, cols, seed, param_scale=1.0, eps=1e-5):
 
 
 def test_static_entry_equals_the_workspace_entry_twice_in_a_row():
-    print("case rows=2048 cols=4096, then rows=300 cols=1024", flush=True)
-    both_entries(2048, 4096, seed=41)                      # fills the whole 16 MiB buffer
+    print("case rows=2048 cols=8192, then rows=300 cols=1024", flush=True)
+    both_entries(2048, 8192, seed=41)                      # fills the whole 16 MiB buffer
     both_entries(300, 1024, seed=42, param_scale=0.25)     # smaller: stale partials beyond its own must not matter
     both_entries(7, 1001, seed=43)                         # the general kernels (width not a multiple of 4)
 
@@ -59,7 +59,7 @@ def test_static_entry_refuses_what_does_not_fit():
     lib = hip.load()
     assert lib.br_hip_layernorm_bwd_static_limit() == 16 << 20
     t = empty(16)
-    rc = lib.br_hip_layernorm_bwd_static(ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 2048, 8192, 1e-5,
+    rc = lib.br_hip_layernorm_bwd_static(ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), ptr(t), 2048, 16384, 1e-5,
                                          1.0, stream())
     assert rc == -5
     assert b"scratch" in lib.br_hip_error_string(rc)
