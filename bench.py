@@ -10,12 +10,12 @@ product path: word script -> word machine -> TensorType -> HIPTensor -> HIP
 kernels.  Inputs and weights are resident in HBM before the timed region.
 
 One JSON line is printed.  Besides the step throughput it carries
-  roofline      the dominant kernel (the direct-to-LDS MFMA GEMM at the h->4h
-                shape of this block) timed on its own with HIP events on the
-                launch stream
+  roofline      the dominant kernel (the direct-to-LDS MFMA GEMM in its
+                weight-gradient form, at the h->4h shape of this block) timed
+                on its own with HIP events on the launch stream
   elementwise   LayerNorm / bias-GELU / log-softmax+NLL kernels in GB/s
-  gemms         every GEMM shape of the block in TFLOP/s, as the backend runs
-                it (fp32 operands staged to fp16) and the kernel alone
+  gemms         every GEMM shape of the block in TFLOP/s (kernel alone, operand
+                and output types as the headline words use them)
   cpu_baseline  the CPU oracle timed on the host cores on a bounded sample
 """
 from __future__ import annotations
@@ -34,10 +34,23 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # dense fp16
-# HBM bytes per launch of the roofline kernel at the roofline shape, from the
-# FETCH_SIZE / WRITE_SIZE counters of rocprofv3, each scaled by what the same
-# counter reads on the copy leg (402.5 MB fetched + 134.2 MB written).
-ROOFLINE_TRAFFIC_BYTES = 536.7e6
+# HBM bytes per launch of the roofline kernel at the roofline shape come from a
+# committed rocprofv3 counter summary (FETCH_SIZE / WRITE_SIZE, each scaled by
+# what the same counter reads on the copy leg), not from this run.
+ROOFLINE_TRAFFIC_PROFILE = os.path.join("profiles", "gemm_dtl_f16_weight_gradient_hbm_traffic.txt")
+
+
+def roofline_traffic():
+    """(bytes per launch, source) from the line `traffic_bytes_per_launch = N`
+    of the committed counter summary; (None, None) when it is absent."""
+    try:
+        with open(os.path.join(ROOT, ROOFLINE_TRAFFIC_PROFILE)) as f:
+            for line in f:
+                if line.lstrip("# ").startswith("traffic_bytes_per_launch"):
+                    return float(line.split("=")[1].split()[0]), ROOFLINE_TRAFFIC_PROFILE
+    except OSError:
+        pass
+    return None, None
 
 H, NH, F, V = 4096, 32, 16384, 250880
 B, T = 4, 512
@@ -164,41 +177,50 @@ def model_leg(args, host, timer):
             "steps": steps}
 
 
-def gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch=1, iters=20, staged=False):
+def gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch=1, iters=20, staged=False, sets=1):
     """Times one product.  staged=True goes through br_hip_gemm_staged the way
     the tensor backend does (fp32 operands converted into a scratch block,
-    conversion time included)."""
+    conversion time included).  sets > 1 rotates that many operand / output
+    sets so that no launch finds its operands in the last-level cache."""
     tt = {hip.F32: torch.float32, hip.F16: torch.float16}
-    a = torch.randn((batch, m * k), device="cuda").to(tt[a_dt])
-    b = torch.randn((batch, n * k), device="cuda").to(tt[b_dt])
-    c = torch.empty((batch, m * n), device="cuda", dtype=tt[c_dt])
+    a = [torch.randn((batch, m * k), device="cuda").to(tt[a_dt]) for _ in range(sets)]
+    b = [torch.randn((batch, n * k), device="cuda").to(tt[b_dt]) for _ in range(sets)]
+    c = [torch.empty((batch, m * n), device="cuda", dtype=tt[c_dt]) for _ in range(sets)]
     lda, ldb = (m if ta else k), (k if tb else n)
     st = timer.stream
-    common = (ta, tb, m, n, k, 1.0, ctypes.c_void_p(a.data_ptr()), a_dt, lda, m * k, ctypes.c_void_p(b.data_ptr()),
-              b_dt, ldb, n * k, 0, ctypes.c_void_p(c.data_ptr()), c_dt, n, m * n, None, batch, hip.GEMM_F16)
+
+    def common(i):
+        j = i % sets
+        return (ta, tb, m, n, k, 1.0, ctypes.c_void_p(a[j].data_ptr()), a_dt, lda, m * k,
+                ctypes.c_void_p(b[j].data_ptr()), b_dt, ldb, n * k, 0, ctypes.c_void_p(c[j].data_ptr()), c_dt, n, m * n,
+                None, batch, hip.GEMM_F16)
     if staged:
         need = hip.load().br_hip_gemm_staged_workspace(ta, tb, m, n, k, a_dt, b_dt, batch)
         ws = torch.empty(max(need, 16), dtype=torch.uint8, device="cuda")
 
         def fn(i):
-            hip.call("br_hip_gemm_staged", *common, ctypes.c_void_p(ws.data_ptr()), need, st)
+            hip.call("br_hip_gemm_staged", *common(i), ctypes.c_void_p(ws.data_ptr()), need, st)
     else:
         def fn(i):
-            hip.call("br_hip_gemm", *common, st)
+            hip.call("br_hip_gemm", *common(i), st)
     sec = timer.run(fn, iters, 3)
     return sec, 2.0 * m * n * k * batch
 
 
 def roofline_leg(hip, timer, torch, full):
-    """Dominant kernel: the direct-to-LDS fp16 MFMA GEMM at the h->4h shape
-    [2048 x 4096] . [16384 x 4096]^T of this block, operands as the tensor
-    backend hands them to it (activations already converted to fp16)."""
+    """Dominant kernel: the direct-to-LDS fp16 MFMA GEMM in its weight-gradient
+    form (both operands row-contiguous, fp32 output), which takes the largest
+    share of the block step (four launches, ~30 % of its time); timed at the
+    h->4h weight gradient dW[16384, 4096] = dy[2048, 16384]^T . x[2048, 4096]
+    with operands as the tensor backend hands them over (already fp16), four
+    operand sets in rotation."""
     f32, f16 = hip.F32, hip.F16
-    sec, flop = gemm_case(hip, timer, torch, 0, 1, N, F, H, f16, f16, f32, iters=30)
-    roof = {"bound": "mfma", "kernel": "gemm_dtl_kernel 256x256x64 (A fp16 [m,k], B fp16 [n,k], C fp32)",
-            "shape": "m=%d n=%d k=%d" % (N, F, H), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
+    sec, flop = gemm_case(hip, timer, torch, 1, 0, F, H, N, f16, f16, f32, iters=32, sets=4)
+    traffic, source = roofline_traffic()
+    roof = {"bound": "mfma", "kernel": "gemm_dtl_kernel 256x256x64 (A fp16 [k,m], B fp16 [k,n], C fp32)",
+            "shape": "m=%d n=%d k=%d" % (F, H, N), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, "us_per_launch": sec * 1e6,
-            "traffic": ROOFLINE_TRAFFIC_BYTES}
+            "traffic": traffic, "traffic_source": source}
     # what a bare MFMA loop (no memory traffic) reaches on this box with operands of zeros and of random values
     scratch = torch.empty(1 << 17, device="cuda")
     probe = ctypes.CDLL(os.path.join(ROOT, "blackriver_amd", "lib", "libbr_probe.so"))
@@ -214,28 +236,37 @@ def roofline_leg(hip, timer, torch, full):
         loop[name] = round(tf.value, 1)
     roof["mfma_loop_tflops"] = loop
     roof["frac_of_random_operand_loop"] = roof["achieved"] / loop["random"]
+    # yardstick, not product: the vendor library's product of the same shape (fp16 in, fp16 out) through torch
+    a = torch.randn((N, F), device="cuda", dtype=torch.float16)
+    b = torch.randn((N, H), device="cuda", dtype=torch.float16)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for i in range(13):
+        if i == 3:
+            e0.record()
+        torch.matmul(a.t(), b)
+    e1.record()
+    torch.cuda.synchronize()
+    roof["vendor_library_tflops_fp16_out"] = round(flop / (e0.elapsed_time(e1) * 1e-3 / 10) / 1e12, 1)
     gemms = []
     if full:
         hd = H // NH
         cases = [
-            ("qkv/dense fwd  y=xW^T", 0, 1, N, H, H, f32, f16, f32, 1),
-            ("h->4h fwd", 0, 1, N, F, H, f32, f16, f32, 1),
-            ("4h->h fwd", 0, 1, N, H, F, f32, f16, f32, 1),
-            ("dx=dy.W (4h->h)", 0, 0, N, F, H, f32, f16, f32, 1),
-            ("dx=dy.W (h->4h)", 0, 0, N, H, F, f32, f16, f32, 1),
-            ("dW=dy^T.x (h->4h)", 1, 0, F, H, N, f32, f32, f32, 1),
-            ("dW=dy^T.x (dense)", 1, 0, H, H, N, f32, f32, f32, 1),
-            ("QK^T", 0, 1, T, T, hd, f32, f32, f32, B * NH),
-            ("PV", 0, 0, T, hd, T, f32, f32, f32, B * NH),
-            ("dV=P^T.dO", 1, 0, T, hd, T, f32, f32, f32, B * NH),
+            ("qkv fwd  y=xW^T", 0, 1, N, 3 * H, H, f16, f16, f16, 1),
+            ("dense fwd", 0, 1, N, H, H, f16, f16, f32, 1),
+            ("h->4h fwd (+GELU epilogue in the step)", 0, 1, N, F, H, f16, f16, f16, 1),
+            ("4h->h fwd", 0, 1, N, H, F, f16, f16, f32, 1),
+            ("dx=dy.W (4h->h)", 0, 0, N, F, H, f16, f16, f16, 1),
+            ("dx=dy.W (h->4h)", 0, 0, N, H, F, f16, f16, f32, 1),
+            ("dW=dy^T.x (h->4h)", 1, 0, F, H, N, f16, f16, f32, 1),
+            ("dW=dy^T.x (dense)", 1, 0, H, H, N, f16, f16, f32, 1),
+            ("QK^T (operator chain only)", 0, 1, T, T, hd, f16, f16, f32, B * NH),
+            ("PV (operator chain only)", 0, 0, T, hd, T, f16, f16, f16, B * NH),
         ]
-        for name, ta, tb, m, n, k, a, b, c, batch in cases:
-            # as the backend runs it (fp32 activations staged to fp16) and the kernel alone on fp16 operands
-            s, fl = gemm_case(hip, timer, torch, ta, tb, m, n, k, a, b, c, batch, iters=10, staged=True)
-            s16, _ = gemm_case(hip, timer, torch, ta, tb, m, n, k, f16, f16, c, batch, iters=10)
-            gemms.append({"name": name, "m": m, "n": n, "k": k, "batch": batch, "us": round(s * 1e6, 1),
-                          "tflops": round(fl / s / 1e12, 1), "kernel_us": round(s16 * 1e6, 1),
-                          "kernel_tflops": round(fl / s16 / 1e12, 1),
+        for name, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch in cases:
+            s16, fl = gemm_case(hip, timer, torch, ta, tb, m, n, k, a_dt, b_dt, c_dt, batch, iters=12, sets=3)
+            gemms.append({"name": name, "m": m, "n": n, "k": k, "batch": batch, "c": "f32" if c_dt == f32 else "f16",
+                          "kernel_us": round(s16 * 1e6, 1), "kernel_tflops": round(fl / s16 / 1e12, 1),
                           "kernel_frac": round(fl / s16 / 1e12 / MFMA_F16_PEAK_TFLOPS, 3)})
     return roof, gemms
 

@@ -26,8 +26,8 @@
 // every other shape.
 //
 // Tile order.  Workgroup ids are first spread so that ids that land on the
-// same XCD (id mod 8) are contiguous, then mapped to tiles in groups of up to
-// 8 x 8 tiles, so the workgroups resident on one XCD at a time share A and B
+// same XCD (id mod 8) are contiguous, then mapped to tiles in blocks of up to
+// 8 x 4 tiles, so the workgroups resident on one XCD at a time share A and B
 // panels in that XCD's L2.
 #pragma once
 
@@ -276,15 +276,21 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch,
     const long long per_batch = (long long)g.tiles_m * g.tiles_n;
     batch = id / per_batch;
     const int rem = (int)(id % per_batch);
-    // groups of GN tile columns; inside a group m varies fastest
-    constexpr int GN = 8;
+    // Panels of GN tile columns; inside a panel, blocks of GM x gn tiles with m
+    // fastest: the ~32 workgroups an XCD runs at a time cover a GM x GN block and
+    // share GM + GN operand strips in its L2 (8 x 4: 12 strips for 32 tiles; a
+    // column-first walk down a tall product would touch 33).
+    const int GM = g.tiles_m < 8 ? g.tiles_m : 8;
+    const int GN = 32 / GM > 4 ? 32 / GM : 4;
     const int group = rem / (GN * g.tiles_m);
     const int first_n = group * GN;
     const int gn = g.tiles_n - first_n < GN ? g.tiles_n - first_n : GN;
     const int in_group = rem - group * GN * g.tiles_m;
-    tm = in_group % g.tiles_m;
-    tn = first_n + in_group / g.tiles_m;
-    (void)gn;
+    const int blk = in_group / (GM * gn);
+    const int within = in_group - blk * GM * gn;
+    const int gm = g.tiles_m - blk * GM < GM ? g.tiles_m - blk * GM : GM;
+    tm = blk * GM + within % gm;
+    tn = first_n + within / gm;
 }
 
 // The K loop.  STAGES register sets: the global loads of K steps t+1 ..
