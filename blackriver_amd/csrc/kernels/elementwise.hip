@@ -401,17 +401,17 @@ __global__ __launch_bounds__(kBlock) void bias_gelu_bwd_kernel(const T* dy, cons
     }
     const int64_t r0 = (int64_t)blockIdx.y * rows_per_block;
     const int64_t r1 = r0 + rows_per_block < rows ? r0 + rows_per_block : rows;
-    // two rows (four loads) in flight per thread; rows are still summed in order
+    // four rows (eight loads) in flight per thread; rows are still summed in order
     int64_t r = r0;
-    for (; r + 2 <= r1; r += 2) {
-        float v[2][VEC], g[2][VEC];
+    for (; r + 4 <= r1; r += 4) {
+        float v[4][VEC], g[4][VEC];
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
+        for (int u = 0; u < 4; u++) {
             VecIO<T, VEC>::load(x + (r + u) * cols + col, v[u]);
             VecIO<T, VEC>::load(dy + (r + u) * cols + col, g[u]);
         }
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
+        for (int u = 0; u < 4; u++) {
 #pragma unroll
             for (int j = 0; j < VEC; j++) g[u][j] *= gelu_grad_one(v[u][j] + b[j]);
             // sum what was stored, i.e. after rounding to the storage type
