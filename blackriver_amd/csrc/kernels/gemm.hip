@@ -419,11 +419,6 @@ int splitk_choice(int64_t m, int64_t n, int64_t k) {
             pick = s;
         }
     }
-    static const char* force = getenv("BR_GEMM_SPLITK");
-    if (force) {
-        const int f = atoi(force);
-        if (f >= 1 && k % (64 * f) == 0) pick = f;
-    }
     return pick;
 }
 

@@ -45,8 +45,6 @@
 
 #include "gemm_mfma16.hpp"
 
-#include <stdlib.h>
-#include <string.h>
 
 namespace brk {
 namespace gemm16 {
@@ -385,13 +383,7 @@ inline DtlPlan dtl_plan(long long m, long long n, long long k, long long batch) 
 
 template <int CT>
 int launch_dtl(const GemmArgs& g, const Problem& p, long long batch, hipStream_t st) {
-    int pick = dtl_plan(g.m, g.n, g.k, batch).config;
-    static const char* force = getenv("BR_GEMM_TILE");
-    if (pick != 3 && force && strcmp(force, "256x256") == 0) pick = 0;
-    if (pick != 3 && force && strcmp(force, "256x128") == 0) pick = 1;
-    if (pick != 3 && force && strcmp(force, "128x128") == 0) pick = 2;
-    if (pick == 0 && force && strcmp(force, "256x256w4") == 0)
-        return launch_dtl_config<CT, 256, 256, 128, 128, 64, 2>(g, p, batch, st);
+    const int pick = dtl_plan(g.m, g.n, g.k, batch).config;
     if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
     if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
     if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);

@@ -386,8 +386,7 @@ __global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restr
 // row walkers each (512 rows in flight chip-wide, 256 partial row pairs).
 constexpr int kBwdWalkers = 2;
 int bwd_parts(int64_t rows) {
-    static const char* e = getenv("BR_LN_PARTS");
-    int64_t p = e ? atoi(e) : 256;
+    int64_t p = 256;
     const int64_t most = (rows + kBwdWalkers - 1) / kBwdWalkers;
     if (p > most) p = most;
     return (int)(p < 1 ? 1 : p);
