@@ -42,6 +42,7 @@
 // operands rows % 8 == 0.  Rows past the end of an operand are redirected to a
 // valid row; their products land in rows / columns of C that are never stored.
 #pragma once
+#include <type_traits>
 
 #include "gemm_mfma16.hpp"
 
@@ -159,6 +160,12 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     long long batch;
     int tm, tn;
     tile_coords(g, batch, tm, tn);
+    // The divisions in tile_coords run on the vector unit although their operands are wave-uniform.  Taking the
+    // results back to scalar registers here keeps everything derived from them (operand tile origins, which the
+    // load statement needs in scalar registers, and the row bases of C) on the scalar unit.
+    tm = __builtin_amdgcn_readfirstlane(tm);
+    tn = __builtin_amdgcn_readfirstlane(tn);
+    batch = __builtin_amdgcn_readfirstlane((int)batch);
     const long long row0 = (long long)tm * BM, col0 = (long long)tn * BN;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -284,26 +291,95 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     //   row = wm*WM + i*32 + (v/4)*8 + (lane/32)*4 + v%4,  col = wn*WN + j*32 + lane%32
     TC* c_base = static_cast<TC*>(g.c) + batch * g.sc;
     TC* c2_base = GELU ? static_cast<TC*>(g.c2) + batch * g.sc : nullptr;
+    if (row0 + BM <= g.m && col0 + BN <= g.n) {
+        // Interior tile: straight-line code without guards, one 32x32 block of accumulators at a time.  A block's
+        // 16 stores leave back to back; when accumulating, the old C of the next block is read before the stores
+        // of this one are issued, so the wait for those reads lets the stores stay in flight.  (In the guarded path
+        // below, a read of C next to each store puts a wait for ALL outstanding memory operations in front of
+        // every element: each store then completes before the next is issued.)  Addresses are a wave-uniform row
+        // base plus one per-lane offset; dtl_applies has checked that the offset fits 32 bits.  The fences keep
+        // the compiler from forming the addresses of all 128 elements ahead of the first store, which takes more
+        // registers than there are.
+        const unsigned lane_bytes = (unsigned)(((lane >> 5) * 4 * g.ldc + (lane & 31)) * (long long)sizeof(TC));
+        const long long tile_at = (row0 + __builtin_amdgcn_readfirstlane(wm) * WM) * g.ldc + col0 +
+                                  __builtin_amdgcn_readfirstlane(wn) * WN;
+        char* const c_tile = reinterpret_cast<char*>(c_base + tile_at);
+        char* const c2_tile = GELU ? reinterpret_cast<char*>(c2_base + tile_at) : nullptr;
+        auto element = [&](char* tile, int blk, int v) {
+            const int i = blk / FN, j = blk % FN;
+            return reinterpret_cast<TC*>(tile + (i * 32 + (v >> 2) * 8 + (v & 3)) * g.ldc * (long long)sizeof(TC) +
+                                         j * 32 * sizeof(TC) + lane_bytes);
+        };
+        float bias[FN];
 #pragma unroll
-    for (int j = 0; j < FN; j++) {
-        const long long col = col0 + wn * WN + j * 32 + (lane & 31);
-        if (col >= g.n) continue;
-        const float bias = g.bias ? g.bias[col] : 0.f;
+        for (int j = 0; j < FN; j++) bias[j] = g.bias ? g.bias[col0 + wn * WN + j * 32 + (lane & 31)] : 0.f;
+        auto interior = [&](auto adds) {
+            constexpr bool ADDS = decltype(adds)::value;
+            // alpha made opaque per form, or the compiler merges the scaling of all 128 elements of the two forms
+            // into one pass ahead of the branch and spills its results
+            float alpha = g.alpha;
+            asm volatile("" : "+v"(alpha));
+            float was[2][16];
+            auto fetch = [&](int blk) {
 #pragma unroll
-        for (int i = 0; i < FM; i++) {
+                for (int v = 0; v < 16; v++) was[blk & 1][v] = c_load<TC>(element(c_tile, blk, v));
+            };
+            if (ADDS) fetch(0);
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const long long row = row0 + wm * WM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
-                if (row < g.m) {
-                    TC* p = c_base + row * g.ldc + col;
-                    float o = g.alpha * acc[i][j][v] + bias;
-                    if (g.accumulate) o += c_load<TC>(p);
-                    c_store<TC>(p, o);
+            for (int blk = 0; blk < FM * FN; blk++) {
+                const int i = blk / FN, j = blk % FN;
+                if (ADDS && blk + 1 < FM * FN) fetch(blk + 1);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    float o = alpha * acc[i][j][v] + bias[j];
+                    if (ADDS) o += was[blk & 1][v];
+                    // A 16-bit C is the rounded copy of this fp32 value, the same bits a later product would make
+                    // of an fp32 C on loading it.  Left alone, the compiler merges the multiply-add and the
+                    // narrowing into one mixed-precision instruction whose result differs in the last place.
+                    if (sizeof(TC) == 2) asm volatile("" : "+v"(o));
+                    c_store<TC>(element(c_tile, blk, v), o);
                     // the activation is taken of the fp32 value, not of its rounded copy
-                    if (GELU) c_store<TC>(c2_base + row * g.ldc + col, gelu_one(o));
+                    if (GELU) c_store<TC>(element(c2_tile, blk, v), gelu_one(o));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        if (g.accumulate) {
+            interior(std::true_type{});
+        } else {
+            interior(std::false_type{});
+        }
+        return;
+    }
+    // Edge tiles: element-wise guards.  The two forms are separate loops so that the plain one holds no read of C.
+    auto guarded = [&](auto adds) {
+#pragma unroll
+        for (int j = 0; j < FN; j++) {
+            const long long col = col0 + wn * WN + j * 32 + (lane & 31);
+            if (col >= g.n) continue;
+            const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const long long row = row0 + wm * WM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                    if (row < g.m) {
+                        TC* p = c_base + row * g.ldc + col;
+                        float o = g.alpha * acc[i][j][v] + bias;
+                        if (decltype(adds)::value) o += c_load<TC>(p);
+                        if (sizeof(TC) == 2) asm volatile("" : "+v"(o));  // as in the interior form
+                        c_store<TC>(p, o);
+                        if (GELU) c_store<TC>(c2_base + row * g.ldc + col, gelu_one(o));
+                    }
                 }
             }
         }
+    };
+    if (g.accumulate) {
+        guarded(std::true_type{});
+    } else {
+        guarded(std::false_type{});
     }
 }
 
@@ -353,7 +429,7 @@ inline bool dtl_applies(const GemmArgs& g, const Problem& p) {
     const long long lim = 1LL << 31;
     const long long a_span = p.a_kstr ? 2 * 64 * g.lda : 2 * 256 * g.lda;
     const long long b_span = p.b_kstr ? 2 * 64 * g.ldb : 2 * 256 * g.ldb;
-    return a_span < lim && b_span < lim;
+    return a_span < lim && b_span < lim && g.ldc < (1LL << 27);
 }
 
 // Tile choice by estimated time: rounds of workgroups over the 256 CUs x the
