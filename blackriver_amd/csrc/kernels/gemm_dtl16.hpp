@@ -149,7 +149,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     using TB = DtlTile<BN, KT, WAVES, B_KSTR>;
     constexpr int kStageBytes = TA::kBytes + TB::kBytes;
     constexpr int kLoads = TA::kPerWave + TB::kPerWave;  // per wave and tile
-    static_assert(STAGES >= 2 && STAGES <= 4, "two to four tile buffers");
+    static_assert(STAGES >= 2 && STAGES <= 6, "two to six tile buffers");
     static_assert(KT == 32 || KT == 64, "K tile of 32 or 64");
     static_assert(FM * FN >= FM + FN, "one LDS fragment read per MFMA slot");
     static_assert(STAGES * kStageBytes <= 160 * 1024, "LDS");
@@ -195,14 +195,20 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     }
 
     const int nk = (int)(g.k / KT);
+    // step `t` of the loop covers K step (t + first) mod nk (see k_walk_start)
+    const int first = (int)(k_walk_start(row0, col0, g.k) / KT);
+    a_src += first * a_step;
+    b_src += first * b_step;
+    int until_wrap = nk - first;  // issues left before the walk returns to K step 0
     auto issue = [&](int tile) {
         const unsigned dst = lds0 + (unsigned)(tile % STAGES) * kStageBytes + (unsigned)wave * 1024u;
 #pragma unroll
         for (int q = 0; q < TA::kPerWave; q++) dtl_load(dst + q * WAVES * 1024, a_off[q], a_src);
 #pragma unroll
         for (int q = 0; q < TB::kPerWave; q++) dtl_load(dst + TA::kBytes + q * WAVES * 1024, b_off[q], b_src);
-        a_src += a_step;
-        b_src += b_step;
+        const bool wraps = --until_wrap == 0;
+        a_src += wraps ? a_step - nk * a_step : a_step;
+        b_src += wraps ? b_step - nk * b_step : b_step;
     };
     auto read_frags = [&](u32x4 (&fa)[FM], u32x4 (&fb)[FN], int tile, int ks) {
         const lds_byte* stage = lds + (tile % STAGES) * kStageBytes;

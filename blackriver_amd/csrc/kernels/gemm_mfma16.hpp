@@ -293,6 +293,20 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch,
     tn = first_n + within / gm;
 }
 
+// Where a tile starts its walk over K (an element index, a multiple of 64; the walk wraps round at the end of K).
+// Workgroups that run side by side would otherwise all read the same 128-byte column of their operand rows at the
+// same time; with row pitches that are large powers of two those lines fall on a few memory channels and the
+// fetches queue behind one another (a [2048 x 4096] by [16384 x 4096] product ran 891 TFLOP/s so, 1150 with the
+// starts spread).  The start depends only on the 256 x 256 block of C the tile lies in and on K, so every kernel and
+// every tile shape in this library sums a given element of C in the same order and produces the same bits; the
+// spread is kept to seven neighbouring columns so that tiles sharing an operand panel still meet in L2.
+__device__ __forceinline__ long long k_walk_start(long long row0, long long col0, long long k) {
+    const long long n64 = k >> 6;
+    if (n64 < 2) return 0;
+    const long long phase = ((row0 >> 8) & 3) + ((col0 >> 8) & 3);
+    return 64 * (phase % n64);
+}
+
 // The K loop.  STAGES register sets: the global loads of K steps t+1 ..
 // t+STAGES are in flight while step t is multiplied, which is what hides HBM /
 // L2 latency.  Two LDS buffers, one barrier per step: a wave can only reach the
@@ -311,11 +325,13 @@ __device__ __forceinline__ void main_loop(const GemmArgs& g, const void* a_base,
     u32x4 ra0[TA::kNumRegs], ra1[TA::kNumRegs], ra2[TA::kNumRegs];
     u32x4 rb0[TB::kNumRegs], rb1[TB::kNumRegs], rb2[TB::kNumRegs];
     const long long nk = (g.k + BK - 1) / BK;
+    const long long first = k_walk_start(row0, col0, g.k) / BK;  // step `s` of the loop covers K step (s + first) mod nk
 
     auto fetch = [&](u32x4 (&xa)[TA::kNumRegs], u32x4 (&xb)[TB::kNumRegs], long long step) {
         if (step < nk) {
-            TA::template fetch<GUARD>(xa, a_base, g.lda, row0, g.m, step * BK, g.k);
-            TB::template fetch<GUARD>(xb, b_base, g.ldb, col0, g.n, step * BK, g.k);
+            const long long at = step + first < nk ? step + first : step + first - nk;
+            TA::template fetch<GUARD>(xa, a_base, g.lda, row0, g.m, at * BK, g.k);
+            TB::template fetch<GUARD>(xb, b_base, g.ldb, col0, g.n, at * BK, g.k);
         }
     };
     auto run = [&](u32x4 (&xa)[TA::kNumRegs], u32x4 (&xb)[TB::kNumRegs], long long step) {
