@@ -296,8 +296,8 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch,
 // Where a tile starts its walk over K (an element index, a multiple of 64; the walk wraps round at the end of K).
 // Workgroups that run side by side would otherwise all read the same 128-byte column of their operand rows at the
 // same time; with row pitches that are large powers of two those lines fall on a few memory channels and the
-// fetches queue behind one another (a [2048 x 4096] by [16384 x 4096] product ran 891 TFLOP/s so, 1150 with the
-// starts spread).  The start depends only on the 256 x 256 block of C the tile lies in and on K, so every kernel and
+// fetches queue behind one another (a [2048 x 4096] by [16384 x 4096] product, run back to back: 1105 TFLOP/s so,
+// 1175 with the starts spread; the other shapes of the BLOOM-7B1 block measure the same either way).  The start depends only on the 256 x 256 block of C the tile lies in and on K, so every kernel and
 // every tile shape in this library sums a given element of C in the same order and produces the same bits; the
 // spread is kept to seven neighbouring columns so that tiles sharing an operand panel still meet in L2.
 __device__ __forceinline__ long long k_walk_start(long long row0, long long col0, long long k) {
