@@ -63,8 +63,8 @@ STEP_GEMM_FLOP = 3.0 * FWD_GEMM_FLOP
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--leg", default="all", choices=["all", "block", "model", "roofline", "elementwise", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--headline-words-only", action="store_true",
@@ -165,7 +165,7 @@ def model_leg(args, host, timer):
     mask[0, tokens - 37:] = 0                       # right padding, 37 of 512 masked
     steps = max(3, args.steps // 4)
     losses = []
-    sec = timer.run(lambda i: losses.append(model.step(ids, mask)), steps, 2)
+    sec = timer.run(lambda i: losses.append(model.step(ids, mask)), steps, max(2, args.warmup // 4))
     assert all(np.isfinite(l) for l in losses), "model step produced a non-finite loss"
     n = batch * tokens
     fwd_block = 2.0 * n * H * (3 * H + H + 2 * F) + 2 * 2.0 * batch * NH * tokens * tokens * (H // NH)
