@@ -126,13 +126,15 @@ def block_leg(args, host, hip, timer):
     env.write("yout_g0", normal((B, T, H), 1.0))
     env.write("mask_", np.ones((B, T), np.int32))
     env.execute("create_operand_buffers create_flash_buffers prepare_batch_flash op.sync")
-    # the backward adds into yout_g in place, so every step starts from a fresh copy.
+    # The operator-chain backward adds into yout_g in place, so each of its steps starts from a fresh copy;
+    # the fused-attention backward leaves yout_g as it is (the next block's gradient is read where it lies).
     # block_step        the reference's operator sequence over the fp32 arena
     # block_step_mixed  the same sequence with product-only operands kept in fp16 buffers;
     #                   it produces the bits block_step produces (tests/test_gpu_block.py)
     # block_step_flash  block_step_mixed with the attention chain as one fused kernel per
     #                   direction (same tolerance against the oracle, not the same bits)
-    step = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step_flash")
+    env.execute("'yout_g' @ 'yout_g0' @ op.copy op.sync")
+    step = env.build("block_step_flash")
     mixed = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step_mixed")
     plain = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step")
     sec = timer.run(lambda i: env.run(step), args.steps, args.warmup)

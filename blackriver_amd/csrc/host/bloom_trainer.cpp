@@ -63,6 +63,12 @@ std::string BloomTrainer::setup_script() const {
         if (flash()) s << "create_flash_buffers\n";
         s << "0 #  " << i << " share_batch_tensors\n";
     }
+    // Activations pass between neighbouring blocks by name, not by copy: block i reads as its xinput the very tensor
+    // block i-1 leaves its output in, and as its yout_g the one block i+1 leaves its input gradient in.  Both are
+    // written again by their owner only after the reader is done with them (a block's backward pass reuses its xa
+    // for the gradient once every later block has finished, forward and backward).
+    for (int i = 2; i <= cfg_.layers; i++) s << i - 1 << " # 'xa' @  " << i << " # 'xinput' !\n";
+    for (int i = 1; i < cfg_.layers; i++) s << i + 1 << " # 'xa' @  " << i << " # 'yout_g' !\n";
     s << "0 #\n";
     return s.str();
 }
@@ -74,12 +80,10 @@ std::string BloomTrainer::step_script() const {
     const char* backward = flash() ? "layer_backward_flash" : mixed() ? "layer_backward_mixed" : "layer_backward_core";
     s << "0 # model_input\n";
     s << "1 # 'xinput' @  0 # 'xinput' @  op.copy   1 # " << forward << "\n";
-    for (int i = 2; i <= n; i++)
-        s << i << " # 'xinput' @  " << i - 1 << " # 'xa' @  op.copy   " << i << " # " << forward << "\n";
+    for (int i = 2; i <= n; i++) s << i << " # " << forward << "\n";  // xinput is block i-1's xa
     s << "0 # 'xa' @  " << n << " # 'xa' @  op.copy   0 # model_head\n";
     s << n << " # 'yout_g' @  0 # 'xc' @  op.copy   " << n << " # " << backward << "\n";
-    for (int i = n - 1; i >= 1; i--)
-        s << i << " # 'yout_g' @  " << i + 1 << " # 'xa' @  op.copy   " << i << " # " << backward << "\n";
+    for (int i = n - 1; i >= 1; i--) s << i << " # " << backward << "\n";  // yout_g is block i+1's xa
     s << "0 # 'xb' @  1 # 'xa' @  op.copy   0 # model_input_backward\n";
     s << "op.sync\n";
     return s.str();
