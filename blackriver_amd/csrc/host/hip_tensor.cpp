@@ -814,6 +814,25 @@ ComputingReturn hip_linear_accumulate(const tensor_t& x, const tensor_t& w, cons
     return OP_OK;
 }
 
+// y = x . w^T + bias + residual in one product (the residual is read in the epilogue); y may be the residual.
+ComputingReturn hip_linear_residual(const tensor_t& x, const tensor_t& w, const tensor_t& bias,
+                                    const tensor_t& residual, const tensor_t& y) {
+    if (!dev(x) || !dev(w) || !dev(bias) || !dev_f32(residual) || x->shape().dim() != 3) return OP_INPUT_ERROR;
+    if (!dev_f32(y)) return OP_OUTPUT_ERROR;
+    const int64_t n = (int64_t)(x->shape()[0] * x->shape()[1]);
+    const int64_t in = (int64_t)x->shape()[2];
+    const int64_t out = (int64_t)w->shape()[0];
+    if ((int64_t)w->shape()[1] != in || (int64_t)bias->items() != out || (int64_t)residual->items() != n * out)
+        return OP_INPUT_ERROR;
+    if ((int64_t)y->items() != n * out) return OP_OUTPUT_ERROR;
+    const int compute = pick_compute({x, w, y});
+    const size_t need = compute == BR_GEMM_F32 ? 0 : br_hip_gemm_staged_workspace(0, 1, n, out, in, code(x), code(w), 1);
+    void* ws = need ? ComputingContext::gemm_staging(0, need) : nullptr;
+    BR_OP(br_hip_linear_residual(x->data(), code(x), w->data(), code(w), bias_f32(bias, 0), residual->data(), y->data(),
+                                 BR_F32, n, out, in, compute, ws, need, stream()));
+    return OP_OK;
+}
+
 ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& scale, const tensor_t& bias,
                                            const tensor_t& var, const tensor_t& y, const tensor_t& dscale,
                                            const tensor_t& dbias, const tensor_t& residual, const tensor_t& din,

@@ -86,6 +86,8 @@ ComputingReturn hip_linear_gelu(const tensor_t& x, const tensor_t& w, const tens
 // op_add(y, ., y) with the addition done in the product's epilogue; the sum is
 // formed from the same fp32 values, so the bits equal the two operators'.
 ComputingReturn hip_linear_accumulate(const tensor_t& x, const tensor_t& w, const tensor_t& bias, const tensor_t& y);
+ComputingReturn hip_linear_residual(const tensor_t& x, const tensor_t& w, const tensor_t& bias,
+                                    const tensor_t& residual, const tensor_t& y);
 // din = layernorm_backward(...) + residual in one pass where the row kernel
 // applies, else the two operators one after the other (din may be residual).
 ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& scale, const tensor_t& bias,

@@ -388,6 +388,11 @@ BR_WORD(LinearAdd,
     Tensors<4> a(stack);
     op_check_word(hip_linear_accumulate(a[0], a[1], a[2], a[3]), "op.linear_add");
 )
+// ( x w b r y -- )   y = x . w^T + b + r        `op.linear` into a temporary + `op.add` of the residual r
+BR_WORD(LinearResidual,
+    Tensors<5> a(stack);
+    op_check_word(hip_linear_residual(a[0], a[1], a[2], a[3], a[4]), "op.linear_residual");
+)
 // ( dy scale bias var y dscale dbias residual din eps -- )   din = dLN + residual
 BR_WORD(LayernormBackwardAdd,
     const float eps = (float)stack.pop_number();
@@ -485,6 +490,7 @@ void load_nn_words(Enviroment& env) {
         {"op.gelu_linear_backward", GeluLinearBackward::creator},
         {"op.linear_add", LinearAdd::creator},
         {"op.linear_gelu", LinearGelu::creator},
+        {"op.linear_residual", LinearResidual::creator},
         {"op.layernorm_backward_add", LayernormBackwardAdd::creator},
         {"op.flash_attn", FlashAttn::creator},
         {"op.flash_attn_backward", FlashAttnBackward::creator},

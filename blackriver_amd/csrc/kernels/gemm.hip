@@ -171,6 +171,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma32_kernel(GemmArgs g) {
         __syncthreads();
     }
     float* c_base = static_cast<float*>(g.c) + batch * g.sc;
+    const float* old_base = g.addend ? static_cast<const float*>(g.addend) + batch * g.sc : c_base;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const long long col = col0 + wn * 64 + j * 32 + lrow;
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma32_kernel(GemmArgs g) {
                 if (row < g.m) {
                     float* p = c_base + row * g.ldc + col;
                     float o = g.alpha * acc[i][j][v] + bias;
-                    if (g.accumulate) o += *p;
+                    if (g.accumulate) o += old_base[row * g.ldc + col];
                     *p = o;
                 }
             }
@@ -194,12 +195,11 @@ __global__ __launch_bounds__(kThreads) void gemm_mfma32_kernel(GemmArgs g) {
 
 long long elem_size(int dtype) { return dtype == BR_F32 ? 4 : 2; }
 
-}  // namespace
-
-extern "C" int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
-                           int a_dtype, int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb,
-                           int64_t stride_b, int accumulate, void* c, int c_dtype, int64_t ldc, int64_t stride_c,
-                           const float* bias, int64_t batch, int compute, br_stream_t stream) {
+// br_hip_gemm with the tensor an accumulating product adds to named separately (null = c itself).
+int gemm_impl(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a, int a_dtype,
+              int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb, int64_t stride_b, int accumulate,
+              const void* addend, void* c, int c_dtype, int64_t ldc, int64_t stride_c, const float* bias, int64_t batch,
+              int compute, br_stream_t stream) {
     if (m < 0 || n < 0 || k < 0 || batch < 0) return BR_ERR_ATTR;
     if (m == 0 || n == 0 || batch == 0) return BR_OK;
     if (!a || !b) return BR_ERR_INPUT;
@@ -219,6 +219,7 @@ extern "C" int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64
     g.sa = stride_a; g.sb = stride_b; g.sc = stride_c;
     g.alpha = alpha;
     g.accumulate = accumulate ? 1 : 0;
+    g.addend = accumulate ? addend : nullptr;
     g.tiles_m = (int)((m + BM - 1) / BM);
     g.tiles_n = (int)((n + BN - 1) / BN);
     const long long blocks = (long long)g.tiles_m * g.tiles_n * batch;
@@ -252,6 +253,16 @@ extern "C" int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64
     p.guarded = !g.vec_a || !g.vec_b || k % 32 != 0 || (ak && m % va != 0) || (bk && n % vb != 0);
     if (compute == BR_GEMM_F16) return gemm16_launch_f16(g, p, batch, st);
     return gemm16_launch_bf16(g, p, batch, st);
+}
+
+}  // namespace
+
+extern "C" int br_hip_gemm(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
+                           int a_dtype, int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb,
+                           int64_t stride_b, int accumulate, void* c, int c_dtype, int64_t ldc, int64_t stride_c,
+                           const float* bias, int64_t batch, int compute, br_stream_t stream) {
+    return gemm_impl(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b, accumulate,
+                     nullptr, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
 }
 
 extern "C" int br_hip_linear_gelu(const void* x, const void* w, const float* bias, void* u, void* y, int dtype,
@@ -372,8 +383,8 @@ int stage_rows(const float* src, long long ld, long long stride, long long rows,
 // atomics.
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4* __restrict__ part, int splits,
                                                             long long mn4, long long n4, float alpha,
-                                                            const float* __restrict__ bias, int accumulate,
-                                                            void* __restrict__ c, int c_dtype, long long ldc) {
+                                                            const float* __restrict__ bias, const void* old,
+                                                            void* c, int c_dtype, long long ldc) {
     for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < mn4;
          i += (long long)gridDim.x * blockDim.x) {
         float4 s = part[i];
@@ -388,18 +399,21 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4* __rest
             for (int j = 0; j < 4; j++) o[j] += bias[col + j];
         }
         if (c_dtype == BR_F32) {
+            // `old`: the tensor an accumulating product adds to (c itself or a tensor laid out like it), else null
             float* dst = static_cast<float*>(c) + row * ldc + col;
+            const float* was = static_cast<const float*>(old) + row * ldc + col;
 #pragma unroll
-            for (int j = 0; j < 4; j++) dst[j] = accumulate ? o[j] + dst[j] : o[j];
+            for (int j = 0; j < 4; j++) dst[j] = old ? o[j] + was[j] : o[j];
         } else if (c_dtype == BR_F16) {
             __half* dst = static_cast<__half*>(c) + row * ldc + col;
+            const __half* was = static_cast<const __half*>(old) + row * ldc + col;
 #pragma unroll
-            for (int j = 0; j < 4; j++) dst[j] = __float2half_rn(accumulate ? o[j] + __half2float(dst[j]) : o[j]);
+            for (int j = 0; j < 4; j++) dst[j] = __float2half_rn(old ? o[j] + __half2float(was[j]) : o[j]);
         } else {
             __hip_bfloat16* dst = static_cast<__hip_bfloat16*>(c) + row * ldc + col;
+            const __hip_bfloat16* was = static_cast<const __hip_bfloat16*>(old) + row * ldc + col;
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                dst[j] = __float2bfloat16(accumulate ? o[j] + __bfloat162float(dst[j]) : o[j]);
+            for (int j = 0; j < 4; j++) dst[j] = __float2bfloat16(old ? o[j] + __bfloat162float(was[j]) : o[j]);
         }
     }
 }
@@ -444,11 +458,12 @@ extern "C" size_t br_hip_gemm_staged_workspace(int trans_a, int trans_b, int64_t
     return need;
 }
 
-extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
-                                  int a_dtype, int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb,
-                                  int64_t stride_b, int accumulate, void* c, int c_dtype, int64_t ldc,
-                                  int64_t stride_c, const float* bias, int64_t batch, int compute, void* workspace,
-                                  size_t workspace_bytes, br_stream_t stream) {
+namespace {
+// br_hip_gemm_staged with the tensor an accumulating product adds to named separately (null = c itself).
+int staged_impl(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a, int a_dtype,
+                int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb, int64_t stride_b, int accumulate,
+                const void* addend, void* c, int c_dtype, int64_t ldc, int64_t stride_c, const float* bias,
+                int64_t batch, int compute, void* workspace, size_t workspace_bytes, br_stream_t stream) {
     const bool f32_a = a_dtype == BR_F32, f32_b = b_dtype == BR_F32;
     const bool sixteen = compute == BR_GEMM_F16 || compute == BR_GEMM_BF16;
     // Stage (and consider splitting K) only when the converted problem meets the
@@ -467,8 +482,8 @@ extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n
             stage = false;
     }
     if (!stage)
-        return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
-                           accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
+        return gemm_impl(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
+                         accumulate, addend, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
     const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
     hipStream_t st = as_stream(stream);
     char* ws = static_cast<char*>(workspace);
@@ -503,10 +518,33 @@ extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n
         const long long mn4 = m * n / 4;
         splitk_reduce_kernel<<<grid_for(mn4, 256, 1 << 14), 256, 0, st>>>(reinterpret_cast<const float4*>(part),
                                                                         splits, mn4, n / 4, alpha, bias,
-                                                                        accumulate ? 1 : 0, c, c_dtype, ldc);
+                                                                        accumulate ? (addend ? addend : c) : nullptr,
+                                                                        c, c_dtype, ldc);
         BR_HIP_LAUNCH_CHECK();
         return BR_OK;
     }
-    return br_hip_gemm(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
-                       accumulate, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
+    return gemm_impl(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b, accumulate,
+                     addend, c, c_dtype, ldc, stride_c, bias, batch, compute, stream);
+}
+}  // namespace
+
+extern "C" int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha, const void* a,
+                                  int a_dtype, int64_t lda, int64_t stride_a, const void* b, int b_dtype, int64_t ldb,
+                                  int64_t stride_b, int accumulate, void* c, int c_dtype, int64_t ldc,
+                                  int64_t stride_c, const float* bias, int64_t batch, int compute, void* workspace,
+                                  size_t workspace_bytes, br_stream_t stream) {
+    return staged_impl(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b,
+                       accumulate, nullptr, c, c_dtype, ldc, stride_c, bias, batch, compute, workspace, workspace_bytes,
+                       stream);
+}
+
+extern "C" int br_hip_linear_residual(const void* x, int x_dtype, const void* w, int w_dtype, const float* bias,
+                                      const void* r, void* y, int y_dtype, int64_t rows, int64_t out, int64_t in,
+                                      int compute, void* workspace, size_t workspace_bytes, br_stream_t stream) {
+    if (rows < 0 || out <= 0 || in <= 0) return BR_ERR_ATTR;
+    if (rows == 0) return BR_OK;
+    if (!x || !w || !r) return BR_ERR_INPUT;
+    if (!y) return BR_ERR_OUTPUT;
+    return staged_impl(0, 1, rows, out, in, 1.0f, x, x_dtype, in, 0, w, w_dtype, in, 0, 1, r, y, y_dtype, out, 0, bias, 1,
+                       compute, workspace, workspace_bytes, stream);
 }

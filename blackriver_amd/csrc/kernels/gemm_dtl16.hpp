@@ -297,6 +297,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     //   row = wm*WM + i*32 + (v/4)*8 + (lane/32)*4 + v%4,  col = wn*WN + j*32 + lane%32
     TC* c_base = static_cast<TC*>(g.c) + batch * g.sc;
     TC* c2_base = GELU ? static_cast<TC*>(g.c2) + batch * g.sc : nullptr;
+    const TC* old_base = g.addend ? static_cast<const TC*>(g.addend) + batch * g.sc : c_base;  // read when accumulating
     if (row0 + BM <= g.m && col0 + BN <= g.n) {
         // Interior tile: straight-line code without guards, one 32x32 block of accumulators at a time.  A block's
         // 16 stores leave back to back; when accumulating, the old C of the next block is read before the stores
@@ -311,6 +312,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                                   __builtin_amdgcn_readfirstlane(wn) * WN;
         char* const c_tile = reinterpret_cast<char*>(c_base + tile_at);
         char* const c2_tile = GELU ? reinterpret_cast<char*>(c2_base + tile_at) : nullptr;
+        char* const old_tile = reinterpret_cast<char*>(const_cast<TC*>(old_base) + tile_at);
         auto element = [&](char* tile, int blk, int v) {
             const int i = blk / FN, j = blk % FN;
             return reinterpret_cast<TC*>(tile + (i * 32 + (v >> 2) * 8 + (v & 3)) * g.ldc * (long long)sizeof(TC) +
@@ -328,7 +330,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
             float was[2][16];
             auto fetch = [&](int blk) {
 #pragma unroll
-                for (int v = 0; v < 16; v++) was[blk & 1][v] = c_load<TC>(element(c_tile, blk, v));
+                for (int v = 0; v < 16; v++) was[blk & 1][v] = c_load<TC>(element(old_tile, blk, v));
             };
             if (ADDS) fetch(0);
 #pragma unroll
@@ -373,7 +375,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                     if (row < g.m) {
                         TC* p = c_base + row * g.ldc + col;
                         float o = g.alpha * acc[i][j][v] + bias;
-                        if (decltype(adds)::value) o += c_load<TC>(p);
+                        if (decltype(adds)::value) o += c_load<TC>(old_base + row * g.ldc + col);
                         if (sizeof(TC) == 2) asm volatile("" : "+v"(o));  // as in the interior form
                         c_store<TC>(p, o);
                         if (GELU) c_store<TC>(c2_base + row * g.ldc + col, gelu_one(o));

@@ -67,6 +67,9 @@ struct GemmArgs {
     // second output of the direct-to-LDS kernel's GELU epilogue: gelu of what
     // goes to c, same layout and type as c (null = plain epilogue)
     void* c2 = nullptr;
+    // what an accumulating product adds to: a tensor laid out like c (same type, leading dimension and batch
+    // stride), read where c is written; null = c itself
+    const void* addend = nullptr;
 };
 
 template <int CT>
@@ -400,6 +403,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_kernel(GemmAr
     // acc[i][j][v] is C[row, col] with
     //   row = wm*WM + i*32 + (v/4)*8 + (lane/32)*4 + v%4,  col = wn*WN + j*32 + lane%32
     TC* c_base = static_cast<TC*>(g.c) + batch * g.sc;
+    const TC* old_base = g.addend ? static_cast<const TC*>(g.addend) + batch * g.sc : c_base;
 #pragma unroll
     for (int j = 0; j < FN; j++) {
         const long long col = col0 + wn * WN + j * 32 + (lane & 31);
@@ -413,7 +417,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_kernel(GemmAr
                 if (row < g.m) {
                     TC* p = c_base + row * g.ldc + col;
                     float o = g.alpha * acc[i][j][v] + bias;
-                    if (g.accumulate) o += c_load<TC>(p);
+                    if (g.accumulate) o += c_load<TC>(old_base + row * g.ldc + col);
                     c_store<TC>(p, o);
                 }
             }

@@ -53,6 +53,7 @@ SIGNATURES = {
     "br_hip_bias_gelu_fwd": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp]),
     "br_hip_bias_gelu_bwd_workspace": (_sz, [_i64, _i64]),
     "br_hip_linear_gelu": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
+    "br_hip_linear_residual": (_int, [_vp, _int, _vp, _int, _vp, _vp, _vp, _int, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "br_hip_bias_gelu_bwd": (_int, [_vp, _vp, _vp, _vp, _vp, _int, _i64, _i64, _f32, _vp, _sz, _vp]),
     "br_hip_transpose_0213": (_int, [_vp, _vp, _int, _i64, _i64, _i64, _i64, _vp]),
     "br_hip_colsum_workspace": (_sz, [_i64, _i64]),

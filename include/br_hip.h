@@ -343,6 +343,19 @@ int br_hip_gemm_staged(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k
 int br_hip_linear_gelu(const void* x, const void* w, const float* bias, void* u, void* y, int dtype,
                        int64_t rows, int64_t out, int64_t in, br_stream_t stream);
 
+/* op_linear followed by op_add of a residual (cuda_tensor.cpp:146-193 and
+ * :206-232; the pair of bloomz-7b/train.words:172-173 and :191-192) in one
+ * product whose epilogue adds the residual:
+ *   y[r, o] = sum_i x[r, i] * w[o, i] + bias[o] + res[r, o]
+ * x [rows, in], w [out, in] (each fp32 or the 16-bit type of `compute`), res and
+ * y [rows, out] of y_dtype, dense; res may be y itself.  The sum is formed as
+ * the two operators form it (product + bias rounded to fp32, then the residual
+ * added), so the result has the bits of the pair.  workspace as for
+ * br_hip_gemm_staged (br_hip_gemm_staged_workspace(0, 1, rows, out, in, ...)). */
+int br_hip_linear_residual(const void* x, int x_dtype, const void* w, int w_dtype, const float* bias,
+                           const void* res, void* y, int y_dtype, int64_t rows, int64_t out, int64_t in,
+                           int compute, void* workspace, size_t workspace_bytes, br_stream_t stream);
+
 /* ---- fused attention --------------------------------------------------- */
 /* The operator chain of bloomz-7b/train.words:154-166 in one kernel:
  *   o = softmax((q . k^T) / sqrt(head_dim) + alibi[h, key] + mask) . v

@@ -429,6 +429,13 @@ def test_linear_add_and_layernorm_backward_add_words_equal_the_operator_pairs(ru
             env.execute("'x' @ 'w' @ 'bias' @ 'tmp' @ op.linear  'acc' @ 'tmp' @ 'y' @ op.add")
             env.execute("'x' @ 'w' @ 'bias' @ 'acc' @ op.linear_add")
             assert np.array_equal(env.read("acc"), env.read("y")), mode
+            # the three-operand form: the residual stays as it is, or is the output itself
+            env.write("acc", acc0)
+            env.execute("'x' @ 'w' @ 'bias' @ 'acc' @ 'din' @ op.linear_residual")
+            assert np.array_equal(env.read("din"), env.read("y")), mode
+            assert np.array_equal(env.read("acc"), acc0), mode
+            env.execute("'x' @ 'w' @ 'bias' @ 'acc' @ 'acc' @ op.linear_residual")
+            assert np.array_equal(env.read("acc"), env.read("y")), mode
 
             env.write("gam", (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32))
             env.write("bet", (0.1 * rng.standard_normal(hidden)).astype(np.float32))
@@ -443,6 +450,31 @@ def test_linear_add_and_layernorm_backward_add_words_equal_the_operator_pairs(ru
             assert np.array_equal(env.read("dgam2"), env.read("dgam")) and np.array_equal(env.read("dbet2"), env.read("dbet"))
         finally:
             env.close()
+
+
+def test_linear_residual_on_a_product_that_is_split_along_k(runtime):
+    """512 rows against a [4096, 16384] weight: few output tiles and a long K, which the backend runs as slices
+    of K summed by a second kernel; the residual then joins in that kernel."""
+    rng = np.random.default_rng(18)
+    rows, out, k = 512, 4096, 16384
+    env = host.Env(1)
+    try:
+        env.execute("'f16' op.gemm_precision")
+        env.execute("1 %d %d 3 'cuda' 'f16' op.create 'x' !  %d %d 2 'cuda' 'f16' op.create 'w' !" % (rows, k, out, k))
+        env.execute("%d 1 'cuda' 'float' op.create 'bias' !" % out)
+        for n in ("tmp", "y", "res", "y2"):
+            env.execute("1 %d %d 3 'cuda' 'float' op.create '%s' !" % (rows, out, n))
+        env.write("x", rng.standard_normal((1, rows, k)).astype(np.float32))
+        env.write("w", (0.02 * rng.standard_normal((out, k))).astype(np.float32))
+        env.write("bias", rng.standard_normal(out).astype(np.float32))
+        res = rng.standard_normal((1, rows, out)).astype(np.float32)
+        env.write("res", res)
+        env.execute("'x' @ 'w' @ 'bias' @ 'tmp' @ op.linear  'tmp' @ 'res' @ 'y' @ op.add")
+        env.execute("'x' @ 'w' @ 'bias' @ 'res' @ 'y2' @ op.linear_residual op.sync")
+        assert np.array_equal(env.read("y2"), env.read("y"))
+        assert np.array_equal(env.read("res"), res)
+    finally:
+        env.close()
 
 
 @pytest.mark.parametrize("mode", ["f16", "f32"])
