@@ -67,6 +67,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--leg", default="all", choices=["all", "block", "model", "roofline", "elementwise", "copy"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--block-words", default="flash", choices=["flash", "mixed", "plain"],
+                    help="with --headline-words-only: which of the three word sets of the block leg to time "
+                         "(for kernel profiles of the operator-chain paths)")
     ap.add_argument("--headline-words-only", action="store_true",
                     help="block leg: time only the word set `value` is quoted on (for kernel profiles of it alone)")
     return ap.parse_args()
@@ -137,6 +140,11 @@ def block_leg(args, host, hip, timer):
     step = env.build("block_step_flash")
     mixed = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step_mixed")
     plain = env.build("'yout_g' @ 'yout_g0' @ op.copy  block_step")
+    if args.headline_words_only and args.block_words != "flash":
+        sec = timer.run(lambda i: env.run(mixed if args.block_words == "mixed" else plain), args.steps, args.warmup)
+        assert np.all(np.isfinite(env.read("xa"))), "block step produced non-finite values"
+        env.close()
+        return sec, None, None
     sec = timer.run(lambda i: env.run(step), args.steps, args.warmup)
     out_flash = env.read("xa")
     assert np.all(np.isfinite(out_flash)), "block step produced non-finite values"
