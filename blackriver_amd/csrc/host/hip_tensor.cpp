@@ -597,7 +597,6 @@ ComputingReturn HIPTensor<DT>::op_linear_backward(tensor_t self, tensor_t x, ten
         return OP_OUTPUT_ERROR;
     const int compute = pick_compute({self, x, weight});
     // bias_g[o] = sum_n dy[n,o]
-    if (DT == DataType::BF16) return OP_TODO_ERROR;
     const size_t need = br_hip_colsum_workspace(n, out);
     void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
     Operand dy{mem_, (int)DT};

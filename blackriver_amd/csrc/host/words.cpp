@@ -299,7 +299,7 @@ BR_WORD(FlashAttn,
                                        f.heads * f.head_dim, f.head_dim, f.tokens * f.heads * f.head_dim,
                                        f.heads * f.head_dim, f.tokens * f.heads * f.head_dim, ComputingContext::stream));
 )
-// ( q k v o dO alibi valid lse dq dk dv -- )   dq, dk, dv: fp32, same layout
+// ( q k v o dO alibi valid lse dq dk dv -- )   dq, dk, dv: fp32 or q's type, same layout
 BR_WORD(FlashAttnBackward,
     Tensors<11> a(stack);
     const tensor_t& q = a[0];
@@ -310,13 +310,14 @@ BR_WORD(FlashAttnBackward,
     br_assert(flash_16(a[1], q) && flash_16(a[2], q) && flash_16(a[3], q) && flash_16(a[4], q),
               "op.flash_attn_backward: k, v, o, dO must match q");
     br_assert(flash_f32(a[7], (size_t)(f.batch * f.heads * f.tokens)), "op.flash_attn_backward: lse");
-    br_assert(flash_f32(a[8], q->items()) && flash_f32(a[9], q->items()) && flash_f32(a[10], q->items()),
-              "op.flash_attn_backward: dq, dk, dv are fp32 tensors of q's size");
+    const bool g32 = flash_f32(a[8], q->items()) && flash_f32(a[9], q->items()) && flash_f32(a[10], q->items());
+    const bool g16 = flash_16(a[8], q) && flash_16(a[9], q) && flash_16(a[10], q);
+    br_assert(g32 || g16, "op.flash_attn_backward: dq, dk, dv are tensors of q's size, all fp32 or all of q's type");
     BR_HIP_CHECK(br_hip_flash_attn_bwd(q->data(), a[1]->data(), a[2]->data(), a[3]->data(), a[4]->data(),
                                        (int)q->dtype(), static_cast<const float*>(a[5]->data()), f.valid,
-                                       static_cast<const float*>(a[7]->data()), delta,
-                                       static_cast<float*>(a[8]->data()), static_cast<float*>(a[9]->data()),
-                                       static_cast<float*>(a[10]->data()), f.batch, f.heads, f.tokens, f.head_dim,
+                                       static_cast<const float*>(a[7]->data()), delta, a[8]->data(), a[9]->data(),
+                                       a[10]->data(), g32 ? BR_F32 : (int)q->dtype(), f.batch, f.heads, f.tokens,
+                                       f.head_dim,
                                        f.heads * f.head_dim, f.head_dim, f.tokens * f.heads * f.head_dim,
                                        f.heads * f.head_dim, f.tokens * f.heads * f.head_dim, ComputingContext::stream));
 )
@@ -341,7 +342,7 @@ BR_WORD(FlashAttnQkv,
                                        3 * hidden, f.head_dim, f.tokens * 3 * hidden, hidden, f.tokens * hidden,
                                        ComputingContext::stream));
 )
-// ( qkv o dO alibi valid lse dqkv -- )   dqkv: fp32 [B, T, 3 * hidden], packed like qkv
+// ( qkv o dO alibi valid lse dqkv -- )   dqkv: [B, T, 3 * hidden] packed like qkv, fp32 or qkv's type
 BR_WORD(FlashAttnQkvBackward,
     Tensors<7> a(stack);
     const tensor_t& o = a[1];
@@ -352,14 +353,18 @@ BR_WORD(FlashAttnQkvBackward,
     br_assert(a[0]->is_cuda() && a[0]->dtype() == o->dtype() && a[0]->items() == 3 * o->items() && flash_16(a[2], o),
               "op.flash_attn_qkv_backward: qkv holds three tensors of o's size and type, dO matches o");
     br_assert(flash_f32(a[5], (size_t)(f.batch * f.heads * f.tokens)), "op.flash_attn_qkv_backward: lse");
-    br_assert(flash_f32(a[6], 3 * o->items()), "op.flash_attn_qkv_backward: dqkv is fp32 of qkv's size");
+    const bool g32 = flash_f32(a[6], 3 * o->items());
+    br_assert(g32 || (a[6]->is_cuda() && a[6]->dtype() == o->dtype() && a[6]->items() == 3 * o->items()),
+              "op.flash_attn_qkv_backward: dqkv has qkv's size and is fp32 or of qkv's type");
     float* delta = static_cast<float*>(ComputingContext::scratch((size_t)(f.batch * f.heads * f.tokens) * sizeof(float)));
     const char* qkv = static_cast<const char*>(a[0]->data());
-    float* g = static_cast<float*>(a[6]->data());
+    char* g = static_cast<char*>(a[6]->data());
+    const int64_t gs = hidden * (g32 ? 4 : 2);  // bytes from dq to dk to dv
     BR_HIP_CHECK(br_hip_flash_attn_bwd(qkv, qkv + 2 * hidden, qkv + 4 * hidden, o->data(), a[2]->data(), (int)o->dtype(),
                                        static_cast<const float*>(a[3]->data()), f.valid,
-                                       static_cast<const float*>(a[5]->data()), delta, g, g + hidden, g + 2 * hidden,
-                                       f.batch, f.heads, f.tokens, f.head_dim, 3 * hidden, f.head_dim,
+                                       static_cast<const float*>(a[5]->data()), delta, g, g + gs, g + 2 * gs,
+                                       g32 ? BR_F32 : (int)o->dtype(), f.batch, f.heads, f.tokens, f.head_dim,
+                                       3 * hidden, f.head_dim,
                                        f.tokens * 3 * hidden, hidden, f.tokens * hidden, ComputingContext::stream));
 )
 

@@ -59,9 +59,10 @@ struct FlashArgs {
     const u16* v;
     u16* o;
     const u16* d_o;
-    float* dq;
-    float* dk;
-    float* dv;
+    void* dq;  // fp32, or the operands' 16-bit type when grad16 is set
+    void* dk;
+    void* dv;
+    int grad16;
     const float* alibi;    // [heads, tokens]
     const int32_t* valid;  // [batch]
     float* lse;            // [batch, heads, tokens]
@@ -537,8 +538,13 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
             const long long off = base + (long long)kk * a.row + (lane & 31);
 #pragma unroll
             for (int db = 0; db < 4; db++) {
-                a.dk[off + db * 32] = dk[db][v] * a.scale;
-                a.dv[off + db * 32] = dv[db][v];
+                if (a.grad16) {
+                    static_cast<u16*>(a.dk)[off + db * 32] = Cvt<CT>::from_f32(dk[db][v] * a.scale);
+                    static_cast<u16*>(a.dv)[off + db * 32] = Cvt<CT>::from_f32(dv[db][v]);
+                } else {
+                    static_cast<float*>(a.dk)[off + db * 32] = dk[db][v] * a.scale;
+                    static_cast<float*>(a.dv)[off + db * 32] = dv[db][v];
+                }
             }
         }
     }
@@ -655,8 +661,8 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
         if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
     }
 
-    if (query < a.tokens) {
-        float* row = a.dq + base + (long long)query * a.row;
+    if (query < a.tokens && !a.grad16) {
+        float* row = static_cast<float*>(a.dq) + base + (long long)query * a.row;
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -664,6 +670,18 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
                 *reinterpret_cast<float4*>(row + db * 32 + g * 8 + half * 4) =
                     make_float4(dq[db][g * 4 + 0] * a.scale, dq[db][g * 4 + 1] * a.scale, dq[db][g * 4 + 2] * a.scale,
                                 dq[db][g * 4 + 3] * a.scale);
+    } else if (query < a.tokens) {
+        u16* row = static_cast<u16*>(a.dq) + base + (long long)query * a.row;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const unsigned lo = (unsigned)Cvt<CT>::from_f32(dq[db][g * 4 + 0] * a.scale) |
+                                    ((unsigned)Cvt<CT>::from_f32(dq[db][g * 4 + 1] * a.scale) << 16);
+                const unsigned hi = (unsigned)Cvt<CT>::from_f32(dq[db][g * 4 + 2] * a.scale) |
+                                    ((unsigned)Cvt<CT>::from_f32(dq[db][g * 4 + 3] * a.scale) << 16);
+                *reinterpret_cast<uint2*>(row + db * 32 + g * 8 + half * 4) = make_uint2(lo, hi);
+            }
     }
 }
 
@@ -717,14 +735,16 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
 }
 
 int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, int dtype,
-                          const float* alibi, const int32_t* valid, const float* lse, float* delta, float* dq,
-                          float* dk, float* dv, int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim,
+                          const float* alibi, const int32_t* valid, const float* lse, float* delta, void* dq,
+                          void* dk, void* dv, int grad_dtype, int64_t batch, int64_t heads, int64_t tokens,
+                          int64_t head_dim,
                           int64_t row_stride, int64_t head_stride, int64_t batch_stride, int64_t o_row_stride,
                           int64_t o_batch_stride, br_stream_t stream) {
     if (batch < 0 || heads <= 0 || tokens <= 0 || head_dim <= 0) return BR_ERR_ATTR;
     if (batch == 0) return BR_OK;
     if (!q || !k || !v || !o || !d_o || !alibi || !valid || !lse) return BR_ERR_INPUT;
     if (!delta || !dq || !dk || !dv) return BR_ERR_OUTPUT;
+    if (grad_dtype != BR_F32 && grad_dtype != dtype) return BR_ERR_TODO;
     if ((dtype != BR_F16 && dtype != BR_BF16) ||
         !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride, o_row_stride,
                         o_batch_stride) || !aligned16(q) ||
@@ -740,6 +760,7 @@ int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     a.dq = dq;
     a.dk = dk;
     a.dv = dv;
+    a.grad16 = grad_dtype != BR_F32;
     a.alibi = alibi;
     a.valid = valid;
     a.lse = const_cast<float*>(lse);

@@ -1090,7 +1090,7 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
     if (rows == 0) return br_hip_fill(out, BR_F32, 0.f, cols, stream);
     if (!x) return BR_ERR_INPUT;
     if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
-    if (dtype != BR_F32 && dtype != BR_F16) return BR_ERR_TODO;
+    if (dtype != BR_F32 && dtype != BR_F16 && dtype != BR_BF16) return BR_ERR_TODO;
     float* partial = (float*)workspace;
     const int vec = dtype == BR_F32 ? 4 : 8;
     if (cols % vec == 0 && aligned16(x) && (cols * (dtype == BR_F32 ? 4 : 2)) % 16 == 0) {
@@ -1100,8 +1100,11 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
         dim3 grid((unsigned)blocks_x, (unsigned)groups);
         if (dtype == BR_F32)
             colsum_partial_vec<float, 4><<<grid, kBlock, 0, st>>>((const float*)x, partial, rows, cols, rpb);
-        else
+        else if (dtype == BR_F16)
             colsum_partial_vec<__half, 8><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
+        else
+            colsum_partial_vec<__hip_bfloat16, 8><<<grid, kBlock, 0, st>>>((const __hip_bfloat16*)x, partial, rows, cols,
+                                                                          rpb);
         BR_HIP_LAUNCH_CHECK();
         return colsum_finish(partial, out, groups, cols, out_scale, st);
     }
@@ -1110,8 +1113,10 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
     dim3 grid((unsigned)((cols + kBlock - 1) / kBlock), (unsigned)groups);
     if (dtype == BR_F32)
         colsum_partial<float><<<grid, kBlock, 0, st>>>((const float*)x, partial, rows, cols, rpb);
-    else
+    else if (dtype == BR_F16)
         colsum_partial<__half><<<grid, kBlock, 0, st>>>((const __half*)x, partial, rows, cols, rpb);
+    else
+        colsum_partial<__hip_bfloat16><<<grid, kBlock, 0, st>>>((const __hip_bfloat16*)x, partial, rows, cols, rpb);
     BR_HIP_LAUNCH_CHECK();
     return colsum_finish(partial, out, groups, cols, out_scale, st);
 }

@@ -81,7 +81,7 @@ SIGNATURES = {
     "br_hip_gemm_staged": (_int, [_int, _int, _i64, _i64, _i64, _f32, _vp, _int, _i64, _i64, _vp, _int, _i64, _i64,
                                   _int, _vp, _int, _i64, _i64, _vp, _i64, _int, _vp, ctypes.c_size_t, _vp]),
     "br_hip_flash_attn_fwd": (_int, [_vp, _vp, _vp, _int, _vp, _vp, _vp, _vp] + [_i64] * 9 + [_vp]),
-    "br_hip_flash_attn_bwd": (_int, [_vp] * 5 + [_int] + [_vp] * 7 + [_i64] * 9 + [_vp]),
+    "br_hip_flash_attn_bwd": (_int, [_vp] * 5 + [_int] + [_vp] * 7 + [_int] + [_i64] * 9 + [_vp]),
     "br_hip_adamw": (_int, [_vp, _int, _vp, _vp, _vp, _vp, _i64, _f32, _f32, _f32, _f32, _f32, _i64, _vp]),
     "br_hip_embedding_gather": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _vp]),
     "br_hip_embedding_scatter_add": (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _f32, _vp]),

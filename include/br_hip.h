@@ -129,7 +129,7 @@ int br_hip_transpose_0213(const void* x, void* y, int elem_bytes, int64_t s0, in
                           int64_t s2, int64_t s3, br_stream_t stream);
 
 /* cudnnReduceTensor(ADD) of cuda_tensor.cpp:738-760: out[c] = sum_r x[r,c]
- * (x fp32 or fp16, out fp32), times out_scale (1 for the plain sum; a
+ * (x fp32, fp16 or bf16, out fp32), times out_scale (1 for the plain sum; a
  * backward pass that carries its activation gradients lifted by a power of two
  * S passes 1/S here to get the bias gradient at its true scale).
  * workspace: br_hip_colsum_workspace bytes. */
@@ -386,15 +386,17 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
  * (cuda_tensor.cpp:830-888), op_softmax_backward (:890-918) and op_qk_backward
  * (:1004-1063) of train.words:217-226 without the [batch, heads, tokens, tokens]
  * tensors: probabilities are recomputed from q, k and lse.  o is the forward's
- * output, d_o its gradient (both `dtype`, o's strides); dq, dk, dv are fp32
- * with the element strides of q, k, v.  delta: fp32 scratch of
+ * output, d_o its gradient (both `dtype`, o's strides); dq, dk, dv are of
+ * grad_dtype (BR_F32, or `dtype`: the gradients rounded once, as the products
+ * of the projection's backward would round them) with the element strides of
+ * q, k, v.  delta: fp32 scratch of
  * batch * heads * tokens entries (receives rowsum(d_o * o)).  Deterministic: one
  * pass accumulates dk / dv per key block, a second one dq per query block.
  * Same shape limits as the forward (BR_ERR_TODO otherwise). */
 int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                           int dtype, const float* alibi, const int32_t* valid, const float* lse,
-                          float* delta, float* dq, float* dk, float* dv, int64_t batch, int64_t heads,
-                          int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
+                          float* delta, void* dq, void* dk, void* dv, int grad_dtype, int64_t batch,
+                          int64_t heads, int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
                           int64_t batch_stride, int64_t o_row_stride, int64_t o_batch_stride,
                           br_stream_t stream);
 

@@ -12,7 +12,7 @@ import torch
 
 import oracle as orc
 from conftest import assert_close
-from gpu_util import BF16, F16, call, dev, empty, host, ptr, stream
+from gpu_util import BF16, F16, F32, call, dev, empty, host, ptr, stream
 from blackriver_amd import hip
 
 pytestmark = pytest.mark.gpu
@@ -131,7 +131,7 @@ def test_flash_backward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype
          *strides, stream())
     gq, gk, gv = (torch.full((b, t, nh, HD), 7.0, device="cuda") for _ in range(3))
     call("br_hip_flash_attn_bwd", ptr(dq_), ptr(dk_), ptr(dv_), ptr(o), ptr(dg), dtype, ptr(alibi), ptr(dvalid),
-         ptr(lse), ptr(delta), ptr(gq), ptr(gk), ptr(gv), *strides, stream())
+         ptr(lse), ptr(delta), ptr(gq), ptr(gk), ptr(gv), F32, *strides, stream())
     assert_close(host(gv), dv_ref, TOL[dtype], "dv")
     assert_close(host(gq), dq_ref, TOL[dtype], "dq")
     assert_close(host(gk), dk_ref, TOL[dtype], "dk")
@@ -141,9 +141,16 @@ def test_flash_backward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype
     h1, h3 = nh * HD, 3 * nh * HD
     at = lambda x, off: ctypes.c_void_p(x.data_ptr() + off)
     call("br_hip_flash_attn_bwd", ptr(packed), at(packed, 2 * h1), at(packed, 4 * h1), ptr(o), ptr(dg), dtype,
-         ptr(alibi), ptr(dvalid), ptr(lse), ptr(delta), ptr(gp), at(gp, 4 * h1), at(gp, 8 * h1), b, nh, t, HD, h3, HD,
-         t * h3, h1, t * h1, stream())
+         ptr(alibi), ptr(dvalid), ptr(lse), ptr(delta), ptr(gp), at(gp, 4 * h1), at(gp, 8 * h1), F32, b, nh, t, HD, h3,
+         HD, t * h3, h1, t * h1, stream())
     assert torch.equal(gp[:, :, 0], gq) and torch.equal(gp[:, :, 1], gk) and torch.equal(gp[:, :, 2], gv)
+    # gradients asked for in the operands' 16-bit type: the fp32 ones rounded once
+    g16 = torch.full((b, t, 3, nh, HD), 7.0, device="cuda", dtype=dq_.dtype)
+    call("br_hip_flash_attn_bwd", ptr(packed), at(packed, 2 * h1), at(packed, 4 * h1), ptr(o), ptr(dg), dtype,
+         ptr(alibi), ptr(dvalid), ptr(lse), ptr(delta), ptr(g16), at(g16, 2 * h1), at(g16, 4 * h1), dtype, b, nh, t, HD,
+         h3, HD, t * h3, h1, t * h1, stream())
+    # (one rounding step away at most: 2^-8 relative covers bf16, 2^-24 absolute the fp16 subnormals)
+    assert bool(((g16.float() - gp).abs() <= gp.abs() * 2.0 ** -8 + 2.0 ** -24).all())
     # keys in the padding receive exactly zero (when the sequence is not empty)
     for bi in range(b):
         if 0 < valid[bi] < t:
