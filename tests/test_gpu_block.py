@@ -14,7 +14,7 @@ import torch
 
 import oracle as orc
 from oracle import bloom_block as blk
-from conftest import assert_close
+from conftest import assert_close, print_ledger
 from blackriver_amd import host
 
 pytestmark = pytest.mark.gpu
@@ -170,6 +170,12 @@ def test_loss_head_against_oracle(runtime, mode):
     env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xb' @ 'lm_g_cpu' @ op.loss_backward")
     assert_close(env.read("lm_g_cpu"), wg_ref - g0, tol, "lm_head_g on the host")
     assert np.array_equal(env.read("xb"), env.read("xa"))
+    # the same tensor again: the plain word adds to what it holds, the overwriting word replaces it
+    once = env.read("lm_g_cpu")
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xb' @ 'lm_g_cpu' @ op.loss_backward")
+    assert_close(env.read("lm_g_cpu"), 2 * once, 1e-6, "lm_head_g on the host, accumulated")
+    env.execute("'xinput' @ 'ids_' @ 'mask_' @ 'lm_head.weight' @ 'all_logits' @ 'xb' @ 'lm_g_cpu' @ op.loss_backward_set")
+    assert np.array_equal(env.read("lm_g_cpu"), once), "op.loss_backward_set left stale contents in a host gradient"
     env.close()
 
 
@@ -607,23 +613,25 @@ def test_block_at_the_full_headline_size_against_oracle(runtime):
 
     def check(step_word, forward_word, what):
         print("  path", what, flush=True)
+        ledger = {}
         env.write("xinput", x)
         env.write("yout_g", dy)
         env.execute("zero_layer_grad")
         env.execute(step_word + " op.sync")
-        assert_close(env.read("xa"), dx_ref, tol, what + ": dx")
+        assert_close(env.read("xa"), dx_ref, tol, what + ": dx", ledger)
         for name, ref in g_ref.items():
             if name.startswith(("query.", "key.", "value.")):
                 continue
-            assert_close(env.read(name).reshape(ref.shape), ref, tol, what + ": " + name)
-        assert_close(env.read("query_key_value.weight_g"), qkv_w, tol, what + ": query_key_value.weight_g")
+            assert_close(env.read(name).reshape(ref.shape), ref, tol, what + ": " + name, ledger)
+        assert_close(env.read("query_key_value.weight_g"), qkv_w, tol, what + ": query_key_value.weight_g", ledger)
         # the key third of the bias gradient is zero up to rounding; query and value thirds are checked
         got_b = env.read("query_key_value.bias_g")
-        assert_close(got_b[:hidden], qkv_b[:hidden], tol, what + ": query bias_g")
-        assert_close(got_b[v_only], qkv_b[v_only], tol, what + ": value bias_g")
+        assert_close(got_b[:hidden], qkv_b[:hidden], tol, what + ": query bias_g", ledger)
+        assert_close(got_b[v_only], qkv_b[v_only], tol, what + ": value bias_g", ledger)
         env.write("xinput", x)
         env.execute(forward_word + " op.sync")
-        assert_close(env.read("xa"), out_ref, tol, what + ": block output")
+        assert_close(env.read("xa"), out_ref, tol, what + ": block output", ledger)
+        print_ledger("C4 block, " + what, ledger)
 
     check("block_step", "layer_forward", "operator words")
     env.execute("create_operand_buffers create_flash_buffers prepare_batch_flash")
