@@ -1,8 +1,11 @@
 #include "bloom_trainer.hpp"
 
+#include <cmath>
 #include <cstring>
 #include <sstream>
+#include <vector>
 
+#include "br_hip.h"
 #include "common.hpp"
 #include "runtime.hpp"
 #include "tensor.hpp"
@@ -166,7 +169,27 @@ float BloomTrainer::step(const int32_t* ids, const int32_t* mask) {
     grad_lift_ = ComputingContext::grad_lift;
     ComputingContext::grad_lift_auto = false;
     ComputingContext::grad_lift = 1.0f;
-    return ComputingContext::last_loss;
+    // Overflow guard.  A lifted 16-bit activation gradient saturates to inf once a per-token gradient exceeds
+    // 65504 / lift, and every gradient further down the backward chain inherits it.  The embedding LayerNorm sits at
+    // the bottom of that chain: its weight gradient (hidden floats) and the loss being finite means no activation
+    // gradient of this step overflowed.
+    const float loss = ComputingContext::last_loss;
+    tensor_t probe = env_.hash().find_tensor("word_embeddings_layernorm.weight_g");
+    std::vector<float> g((size_t)cfg_.hidden);
+    br_assert(probe->items() == g.size(), "embedding LayerNorm gradient has an unexpected size");
+    if (br_hip_memcpy_d2h(g.data(), probe->data(), g.size() * sizeof(float), ComputingContext::stream) != 0)
+        br_panic("BloomTrainer::step: reading back the embedding LayerNorm gradient failed");
+    ComputingContext::sync();
+    bool finite = std::isfinite(loss);
+    for (float v : g) finite = finite && std::isfinite(v);
+    if (!finite) {
+        std::ostringstream why;
+        why << "BloomTrainer::step: non-finite loss or gradient (loss " << loss << ", gradient lift " << grad_lift_
+            << "); with 16-bit products lower the lift by a power of two with `<S> op.grad_lift`, or run the products "
+               "in bf16 / fp32";
+        br_panic(why.str().c_str());
+    }
+    return loss;
 }
 
 }  // namespace br

@@ -487,6 +487,9 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
     // zero it right before (ComputingContext::loss_head_overwrite) gets the
     // first chunk written instead of added, which saves clearing and re-reading
     // a [vocab, hidden] tensor
+    // (a host-resident gradient goes through the zeroed staging buffer either way;
+    // in overwrite mode the staged sum is assigned to it instead of added)
+    const bool overwrite_host = ComputingContext::loss_head_overwrite && !lm_head_g->is_cuda();
     bool overwrite = ComputingContext::loss_head_overwrite && lm_head_g->is_cuda();
     if (overwrite && count == 0) BR_OP(br_hip_fill(d_wg, BR_F32, 0.f, vocab * hidden, stream()));
     for (int64_t r0 = 0; r0 < n && count > 0; r0 += cap) {
@@ -550,7 +553,11 @@ TransformerComputing::loss_result_t HIPTensor<DT>::op_loss_backward(tensor_t sel
             const size_t cnt = std::min(per, all - off);
             BR_OP(br_hip_memcpy_d2h(bounce, d_wg + off, cnt * sizeof(float), stream()));
             ComputingContext::sync();
-            for (size_t i = 0; i < cnt; i++) host_g[off + i] += bounce[i];
+            if (overwrite_host) {
+                memcpy(host_g + off, bounce, cnt * sizeof(float));
+            } else {
+                for (size_t i = 0; i < cnt; i++) host_g[off + i] += bounce[i];
+            }
         }
         hip_tensor_free(staging);
     }

@@ -315,10 +315,22 @@ void Enviroment::run_(DaG* dag) {
     }
 }
 
+// The gradient lift is a setting of the (process-wide) computing context that
+// scripts change with op.grad_lift; a new environment starts from "off", and
+// one that goes away takes its setting with it.
+static void reset_context_settings() {
+    ComputingContext::grad_lift = 1.0f;
+    ComputingContext::grad_lift_auto = false;
+    ComputingContext::loss_head_overwrite = false;
+}
+
 Enviroment::Enviroment(const int hash_num) : target_(0) {
     hashes_.resize(hash_num > 0 ? (size_t)hash_num : 1);
     load_base_words();
+    reset_context_settings();
 }
+
+Enviroment::~Enviroment() { reset_context_settings(); }
 
 void Enviroment::insert_native_word(const std::string& name, NativeCreator* fn) {
     if (native_words_.count(name)) br_panic("Can't insert native word with same name!");

@@ -212,7 +212,7 @@ private:
 
 struct Enviroment {
     explicit Enviroment(const int hash_num = 1);
-    ~Enviroment() {}
+    ~Enviroment();
 
     void insert_native_word(const std::string& name, NativeCreator* fn);
     // Registers a fusion: wherever a linked program runs the native words

@@ -229,9 +229,12 @@ BR_WORD(LossBackward, Tensors<7> a(stack); a[0]->op_loss_backward(a[0], a[1], a[
 // the clearing pass and the re-read of a [vocab, hidden] tensor (extension)
 BR_WORD(LossBackwardSet,
     Tensors<7> a(stack);
-    ComputingContext::loss_head_overwrite = true;
+    // the flag is this call's only, also when the operator leaves by an exception
+    struct Overwrite {
+        Overwrite() { ComputingContext::loss_head_overwrite = true; }
+        ~Overwrite() { ComputingContext::loss_head_overwrite = false; }
+    } guard;
     a[0]->op_loss_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6]);
-    ComputingContext::loss_head_overwrite = false;
 )
 // ( dy scale bias var y dscale dbias din eps -- )
 BR_WORD(LayernormBackward,
