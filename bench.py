@@ -85,12 +85,18 @@ class Timer:
         hip.call("br_hip_event_create", ctypes.byref(self.e0))
         hip.call("br_hip_event_create", ctypes.byref(self.e1))
 
-    def run(self, fn, iters, warmup):
+    def run(self, fn, iters, warmup, blocker=None):
+        """Seconds per call of fn.  `blocker` enqueues a long kernel right before
+        the first event: the timed launches then pile up behind it in the queue and
+        run back to back, so that for kernels of a few microseconds the time
+        between the events is kernel time and not the host's launch rate."""
         if self.device_sync:
             self.device_sync()   # buffers made on another stream are complete
         for i in range(warmup):
             fn(i)
         self.hip.call("br_hip_stream_sync", self.stream)
+        if blocker:
+            blocker()
         self.hip.call("br_hip_event_record", self.e0, self.stream)
         for i in range(iters):
             fn(i)
@@ -297,6 +303,13 @@ def elementwise_leg(hip, timer, torch):
         out[name] = {"us": round(sec * 1e6, 2), "GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3),
                      "algorithmic_MB": round(nbytes / 1e6, 2)}
 
+    # ~1.5 ms of fill kernels: longer than the host needs to enqueue 200 launches
+    block_buf = torch.empty(1 << 30, device="cuda")
+
+    def blocker():
+        for _ in range(2):
+            hip.call("br_hip_fill", vp(block_buf), hip.F32, 0.0, block_buf.numel(), st)
+
     nb = 8
     rows, cols = 2048, 4096
     xs = [torch.randn((rows, cols), device="cuda") for _ in range(nb)]
@@ -308,13 +321,17 @@ def elementwise_leg(hip, timer, torch):
     mean, var = torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda")
     dg, db = torch.empty(cols, device="cuda"), torch.empty(cols, device="cuda")
     sec = timer.run(lambda i: hip.call("br_hip_layernorm_fwd", vp(xs[i % nb]), vp(g), vp(b), vp(ys[i % nb]), vp(mean),
-                                       vp(var), rows, cols, 1e-5, st), 200, 10)
+                                       vp(var), rows, cols, 1e-5, st), 200, 10, blocker)
     rec("layernorm_fwd [2048,4096] f32", sec, 2 * rows * cols * 4)
     ws = torch.empty(lib.br_hip_layernorm_bwd_workspace(rows, cols), dtype=torch.uint8, device="cuda")
     sec = timer.run(lambda i: hip.call("br_hip_layernorm_bwd", vp(dys[i % nb]), vp(ys[i % nb]), vp(g), vp(b), vp(var),
                                        vp(dg), vp(db), vp(dxs[i % nb]), rows, cols, 1e-5, 1.0, vp(ws), ws.numel(), st),
-                    200, 10)
+                    200, 10, blocker)
     rec("layernorm_bwd [2048,4096] f32", sec, 3 * rows * cols * 4)
+    # yardstick: a plain copy of the same tensors (same rotation, same timing method)
+    sec = timer.run(lambda i: hip.call("br_hip_cast", vp(xs[i % nb]), hip.F32, vp(ys[i % nb]), hip.F32, rows * cols, st),
+                    200, 10, blocker)
+    rec("copy [2048,4096] f32 (yardstick)", sec, 2 * rows * cols * 4)
     del xs, ys, dys, dxs
 
     rows, cols = 2048, 16384
@@ -324,13 +341,13 @@ def elementwise_leg(hip, timer, torch):
     bias = torch.randn(cols, device="cuda") * 0.02
     dbias = torch.empty(cols, device="cuda")
     sec = timer.run(lambda i: hip.call("br_hip_bias_gelu_fwd", vp(xs[i % nb]), vp(bias), vp(ys[i % nb]), hip.F16, rows,
-                                       cols, st), 200, 10)
+                                       cols, st), 200, 10, blocker)
     rec("bias_gelu_fwd [2048,16384] f16", sec, 2 * rows * cols * 2)
     ws = torch.empty(lib.br_hip_bias_gelu_bwd_workspace(rows, cols), dtype=torch.uint8, device="cuda")
     sec = timer.run(lambda i: hip.call("br_hip_bias_gelu_bwd", vp(dys[i % nb]), vp(xs[i % nb]), vp(bias), vp(ys[i % nb]),
-                                       vp(dbias), hip.F16, rows, cols, 1.0, vp(ws), ws.numel(), st), 200, 10)
+                                       vp(dbias), hip.F16, rows, cols, 1.0, vp(ws), ws.numel(), st), 200, 10, blocker)
     rec("bias_gelu_bwd [2048,16384] f16 (+dbias)", sec, 3 * rows * cols * 2)
-    del xs, ys, dys
+    del xs, ys, dys, block_buf
 
     rows, vocab = 2048, V
     logits = torch.randn((rows, vocab), device="cuda") * 2.0
@@ -396,7 +413,59 @@ def cpu_baseline_leg():
     sec = time.perf_counter() - t0
     return {"value": b * t / sec, "unit": "tokens/s", "cores": orc.threads(), "kind": "port",
             "sample": "one step of the same block (H=4096, 32 heads, FFN 16384) fwd+bwd at batch %d x %d tokens, fp32 "
-                      "storage with fp64 accumulation, %.1f s of CPU work" % (b, t, sec)}
+                      "storage with fp64 accumulation, %.1f s of CPU work" % (b, t, sec),
+            "kernels": cpu_kernel_rows(orc)}
+
+
+def cpu_kernel_rows(orc):
+    """The memory-bound kernels of configurations C1-C3 on the host cores (the
+    oracle's restatements, all threads): wall time and the same algorithmic
+    bytes per second the GPU rows quote.  C1 and C2 run at full size, C3 on a
+    64-row sample of its 2048 rows (1 MB per row; the kernels are row-parallel,
+    so the rate carries over).  A baseline to read the GPU rows against, never
+    a target."""
+    rng = np.random.default_rng(0)
+    rows = {}
+
+    def timed(fn, reps=3):
+        fn()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        return (time.perf_counter() - t0) / reps
+
+    def rec(name, sec, nbytes, note=""):
+        rows[name] = {"us": round(sec * 1e6, 1), "GB/s": round(nbytes / sec / 1e9, 2), "algorithmic_MB": round(nbytes / 1e6, 2)}
+        if note:
+            rows[name]["sample"] = note
+
+    r, c = 2048, 4096
+    x = rng.standard_normal((1, r, c)).astype(np.float32)
+    g = (1 + 0.02 * rng.standard_normal(c)).astype(np.float32)
+    bt = (0.02 * rng.standard_normal(c)).astype(np.float32)
+    dy = rng.standard_normal((1, r, c)).astype(np.float32)
+    y, _, var = orc.layernorm_fwd(x, g, bt, 1e-5)
+    rec("layernorm_fwd [2048,4096] f32", timed(lambda: orc.layernorm_fwd(x, g, bt, 1e-5)), 2 * r * c * 4)
+    rec("layernorm_bwd [2048,4096] f32", timed(lambda: orc.layernorm_bwd(dy, y, g, bt, var, 1e-5)), 3 * r * c * 4)
+    r, c = 2048, 16384
+    x = (1.5 * rng.standard_normal((r, c))).astype(np.float32)
+    bias = (0.02 * rng.standard_normal(c)).astype(np.float32)
+    dy = rng.standard_normal((r, c)).astype(np.float32)
+    # the CPU path stores fp32 (the reference has no 16-bit host type); bytes are counted as the GPU row counts
+    # them (2 B per element), so the two GB/s columns compare like with like
+    rec("bias_gelu_fwd [2048,16384]", timed(lambda: orc.bias_gelu_fwd(x, bias)), 2 * r * c * 2, "fp32 storage on the host")
+    rec("bias_gelu_bwd [2048,16384] (+dbias)", timed(lambda: orc.bias_gelu_bwd(dy, x, bias)), 3 * r * c * 2,
+        "fp32 storage on the host")
+    r, v = 64, V
+    logits = (2.0 * rng.standard_normal((r, v))).astype(np.float32)
+    target = rng.integers(0, v, r).astype(np.int32)
+    keep = (rng.random(r) < 0.9).astype(np.int32)
+    note = "64 of the 2048 rows"
+    rec("logsoftmax_nll_fwd [2048,250880] f32", timed(lambda: orc.logsoftmax_nll(logits, target, keep, False)), r * v * 4, note)
+    both = timed(lambda: orc.logsoftmax_nll(logits, target, keep, True))
+    rec("logsoftmax_nll_fwd+bwd [2048,250880] f32", both, 3 * r * v * 4, note + "; the host routine computes the loss and "
+        "the gradient in one call")
+    return rows
 
 
 def main():

@@ -46,7 +46,7 @@ HIPCC_FLAGS = [
     # keep the compiler from forming packed-fp32 instructions
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("BR_HIPCC_EXTRA", "").split()   # e.g. BR_HIPCC_EXTRA="-DBR_STREAM=0" for an A/B build
 CXX_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-maybe-uninitialized", "-I" + INCLUDE, "-I" + HOST_DIR]
 
 

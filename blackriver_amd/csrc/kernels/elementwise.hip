@@ -64,10 +64,11 @@ __global__ __launch_bounds__(kBlock) void cast_x8_kernel(const S* __restrict__ s
     for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n8; i += stride) {
         float f[8];
         if constexpr (sizeof(S) == 4) {
-            const float4 a = reinterpret_cast<const float4*>(src)[2 * i], b = reinterpret_cast<const float4*>(src)[2 * i + 1];
+            const float4 a = load_stream(reinterpret_cast<const float4*>(src) + 2 * i),
+                         b = load_stream(reinterpret_cast<const float4*>(src) + 2 * i + 1);
             f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
         } else {
-            const uint4 raw = reinterpret_cast<const uint4*>(src)[i];
+            const uint4 raw = load_stream(reinterpret_cast<const uint4*>(src) + i);
             const unsigned w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -289,11 +290,11 @@ struct VecIO;
 template <>
 struct VecIO<float, 4> {
     static __device__ __forceinline__ void load(const float* p, float (&f)[4]) {
-        const float4 v = *reinterpret_cast<const float4*>(p);
+        const float4 v = load_stream(reinterpret_cast<const float4*>(p));
         f[0] = v.x; f[1] = v.y; f[2] = v.z; f[3] = v.w;
     }
     static __device__ __forceinline__ void store(float* p, const float (&f)[4]) {
-        *reinterpret_cast<float4*>(p) = make_float4(f[0], f[1], f[2], f[3]);
+        store_stream(reinterpret_cast<float4*>(p), make_float4(f[0], f[1], f[2], f[3]));
     }
     // store, and leave in f exactly the values that were stored
     static __device__ __forceinline__ void store_rounded(float* p, float (&f)[4]) { store(p, f); }
@@ -301,10 +302,10 @@ struct VecIO<float, 4> {
 template <>
 struct VecIO<__half, 8> {
     static __device__ __forceinline__ void load(const __half* p, float (&f)[8]) {
-        unpack8(*reinterpret_cast<const half8*>(p), f);
+        unpack8(load_stream(reinterpret_cast<const half8*>(p)), f);
     }
     static __device__ __forceinline__ void store(__half* p, const float (&f)[8]) {
-        *reinterpret_cast<half8*>(p) = pack8(f);
+        store_stream(reinterpret_cast<half8*>(p), pack8(f));
     }
     // The compiler is free to fuse the producing multiply into the fp16
     // conversion (v_fma_mixlo_f16: one rounding) for one use and not for
@@ -315,7 +316,7 @@ struct VecIO<__half, 8> {
         uint4 u = __builtin_bit_cast(uint4, pack8(f));
         asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w));
         const half8 h = __builtin_bit_cast(half8, u);
-        *reinterpret_cast<half8*>(p) = h;
+        store_stream(reinterpret_cast<half8*>(p), h);
         unpack8(h, f);
     }
 };
@@ -323,7 +324,7 @@ struct VecIO<__half, 8> {
 template <>
 struct VecIO<__hip_bfloat16, 8> {
     static __device__ __forceinline__ void load(const __hip_bfloat16* p, float (&f)[8]) {
-        unpack(*reinterpret_cast<const uint4*>(p), f);
+        unpack(load_stream(reinterpret_cast<const uint4*>(p)), f);
     }
     static __device__ __forceinline__ void unpack(const uint4& u, float (&f)[8]) {
         const unsigned w[4] = {u.x, u.y, u.z, u.w};
@@ -342,12 +343,12 @@ struct VecIO<__hip_bfloat16, 8> {
         return make_uint4(w[0], w[1], w[2], w[3]);
     }
     static __device__ __forceinline__ void store(__hip_bfloat16* p, const float (&f)[8]) {
-        *reinterpret_cast<uint4*>(p) = pack(f);
+        store_stream(reinterpret_cast<uint4*>(p), pack(f));
     }
     static __device__ __forceinline__ void store_rounded(__hip_bfloat16* p, float (&f)[8]) {
         uint4 u = pack(f);
         asm volatile("" : "+v"(u.x), "+v"(u.y), "+v"(u.z), "+v"(u.w));
-        *reinterpret_cast<uint4*>(p) = u;
+        store_stream(reinterpret_cast<uint4*>(p), u);
         unpack(u, f);
     }
 };

@@ -42,7 +42,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_regs(const float* __restrict__ 
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int idx = threadIdx.x + i * kBlock;
-        v[i] = idx < cols4 ? xr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+        v[i] = idx < cols4 ? load_stream(xr + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     float s[1] = {0.f};
 #pragma unroll
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_regs(const float* __restrict__ 
             o.z = (v[i].z - mean) * rstd * g.z + b.z;
             o.w = (v[i].w - mean) * rstd * g.w + b.w;
             store4_as16(y16, row * cols4 + idx, o);
-            yr[idx] = o;
+            store_stream(yr + idx, o);
         }
     }
 }
@@ -144,16 +144,20 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
         acc_b[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     float4 d[VPT], xh[VPT], nd[VPT], nxh[VPT];
-    // rows past the end read as dy = 0, y = beta: they add nothing to any sum
+    // rows past the end read as dy = 0, y = 0: they add nothing to any sum
     auto request = [&](float4 (&rd)[VPT], float4 (&ry)[VPT], int64_t row) {
-        const float4* dyr = reinterpret_cast<const float4*>(dy) + row * cols4;
-        const float4* yr = reinterpret_cast<const float4*>(y) + row * cols4;
 #pragma unroll
         for (int i = 0; i < VPT; i++) {
             const int idx = tid + i * kWalker;
             const bool ok = idx < cols4 && row < rows;
-            rd[i] = ok ? dyr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-            ry[i] = ok ? yr[idx] : b[i];
+            // Dead lanes (columns or rows past the end) load element 0 and replace it by zeros: with dy = 0 they
+            // add nothing to any sum whatever xhat comes out of y = 0.  (A choice `ok ? yr[idx] : b[i]` is turned
+            // into a choice between two addresses, which puts b into private memory to give it one.)
+            const int64_t at = ok ? row * cols4 + idx : 0;
+            const float4 vd = load_stream(reinterpret_cast<const float4*>(dy) + at);
+            const float4 vy = load_stream(reinterpret_cast<const float4*>(y) + at);
+            rd[i] = ok ? vd : make_float4(0.f, 0.f, 0.f, 0.f);
+            ry[i] = ok ? vy : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
     const int64_t stride = (int64_t)gridDim.x * GROUPS;
@@ -176,7 +180,7 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
 #pragma unroll
             for (int i = 0; i < VPT; i++) {
                 const int idx = tid + i * kWalker;
-                res[i] = (idx < cols4 && live) ? rr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+                res[i] = (idx < cols4 && live) ? load_stream(rr + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
             }
         }
         float s[2] = {0.f, 0.f};
@@ -224,7 +228,7 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
                     asm volatile("" : "+v"(o.x), "+v"(o.y), "+v"(o.z), "+v"(o.w));
                     o.x += res[i].x; o.y += res[i].y; o.z += res[i].z; o.w += res[i].w;
                 }
-                dxr[idx] = o;
+                dxr[idx] = o;  // an ordinary store: measured faster here than the streaming form
             }
         }
 #pragma unroll
@@ -519,13 +523,15 @@ static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamm
         const float inv = 1.0f / (float)cols;
         const int vpt = (cols4 + kBlock - 1) / kBlock;
         constexpr int G = kBwdWalkers;
-#define BR_LN_BWD(V)                                                                                              \
-    ln_bwd_regs<V, G><<<parts, kWalker * G, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, \
+#define BR_LN_BWD(V, W)                                                                                           \
+    ln_bwd_regs<V, W><<<parts, kWalker * W, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, \
                                                      inv, residual)
-        if (vpt <= 1) BR_LN_BWD(1);
-        else if (vpt <= 2) BR_LN_BWD(2);
-        else if (vpt <= 4) BR_LN_BWD(4);
-        else BR_LN_BWD(8);
+        // Rows wider than 4096 floats keep 8 quads per thread in flight twice over; with two walkers (512
+        // threads, 256 registers per wave) that spills, so they run one walker per workgroup.
+        if (vpt <= 1) BR_LN_BWD(1, G);
+        else if (vpt <= 2) BR_LN_BWD(2, G);
+        else if (vpt <= 4) BR_LN_BWD(4, G);
+        else BR_LN_BWD(8, 1);
 #undef BR_LN_BWD
         BR_HIP_LAUNCH_CHECK();
         if (aligned16(dgamma) && aligned16(dbeta))

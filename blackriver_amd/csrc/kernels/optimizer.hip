@@ -52,12 +52,12 @@ __global__ __launch_bounds__(kBlock) void adamw_kernel(T* param, float* master, 
     const int64_t stride = (int64_t)gridDim.x * kBlock * VEC;
     for (int64_t base = ((int64_t)blockIdx.x * kBlock + threadIdx.x) * VEC; base < n; base += stride) {
         if (VEC == 4) {
-            const float4 g4 = *reinterpret_cast<const float4*>(grad + base);
-            float4 m4 = *reinterpret_cast<const float4*>(m + base);
-            float4 v4 = *reinterpret_cast<const float4*>(v + base);
+            const float4 g4 = load_stream(reinterpret_cast<const float4*>(grad + base));
+            float4 m4 = load_stream(reinterpret_cast<const float4*>(m + base));
+            float4 v4 = load_stream(reinterpret_cast<const float4*>(v + base));
             float p[4];
             if (master) {
-                const float4 p4 = *reinterpret_cast<const float4*>(master + base);
+                const float4 p4 = load_stream(reinterpret_cast<const float4*>(master + base));
                 p[0] = p4.x; p[1] = p4.y; p[2] = p4.z; p[3] = p4.w;
             } else {
 #pragma unroll
@@ -68,9 +68,9 @@ __global__ __launch_bounds__(kBlock) void adamw_kernel(T* param, float* master, 
             p[2] = adamw_one(p[2], g4.z, m4.z, v4.z, a);
             p[3] = adamw_one(p[3], g4.w, m4.w, v4.w, a);
             asm volatile("" : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]));
-            *reinterpret_cast<float4*>(m + base) = m4;
-            *reinterpret_cast<float4*>(v + base) = v4;
-            if (master) *reinterpret_cast<float4*>(master + base) = make_float4(p[0], p[1], p[2], p[3]);
+            store_stream(reinterpret_cast<float4*>(m + base), m4);
+            store_stream(reinterpret_cast<float4*>(v + base), v4);
+            if (master) store_stream(reinterpret_cast<float4*>(master + base), make_float4(p[0], p[1], p[2], p[3]));
 #pragma unroll
             for (int j = 0; j < 4; j++) param[base + j] = from_f32<T>(p[j]);
         } else {

@@ -271,7 +271,7 @@ __device__ __forceinline__ float row_logsumexp(const float* __restrict__ lr, int
         const float4* l4 = reinterpret_cast<const float4*>(lr);
         const int64_t n4 = vocab / 4;
         for (int64_t i = threadIdx.x; i < n4; i += kVBlock) {
-            const float4 v = l4[i];
+            const float4 v = load_stream(l4 + i);
             const float m4 = fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w));
             if (m4 > t.m) {
                 t.s *= __expf(t.m - m4);  // exp(-inf) = 0 on the first vector
@@ -342,7 +342,7 @@ template <typename OUT>
 __device__ __forceinline__ void store4(OUT* p, float a, float b, float c, float d);
 template <>
 __device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
-    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+    store_stream(reinterpret_cast<float4*>(p), make_float4(a, b, c, d));
 }
 template <>
 __device__ __forceinline__ void store4<__half>(__half* p, float a, float b, float c, float d) {
@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kVBlock) void nll_bwd_kernel(const float* logits, c
         const float4* l4 = reinterpret_cast<const float4*>(lr);
         const int64_t t4 = t >> 2;
         for (int64_t i = threadIdx.x; i < vocab / 4; i += kVBlock) {
-            const float4 v = l4[i];
+            const float4 v = load_stream(l4 + i);
             float e[4] = {__expf(v.x - l), __expf(v.y - l), __expf(v.z - l), __expf(v.w - l)};
             if (i == t4) e[t & 3] -= 1.0f;
             store4<OUT>(dr + i * 4, e[0] * scale, e[1] * scale, e[2] * scale, e[3] * scale);
