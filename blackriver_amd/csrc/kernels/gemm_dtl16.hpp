@@ -58,6 +58,12 @@ typedef __attribute__((address_space(3))) unsigned char lds_byte;
 // rejects it in a clobber list; it holds no compiler-owned value here because
 // these kernels contain none of the operations the compiler itself routes
 // through M0 (indexed register moves, GWS, messages, lane-indexed reads).
+// INVARIANT for whoever adds a kernel that calls dtl_load (or code to one that
+// does): it must not contain dynamically indexed register arrays (every array
+// index a compile-time constant after unrolling), LDS instructions that take M0
+// on this target (none do on gfx9 and later), s_sendmsg, GWS or ds_bpermute-free
+// lane-indexed reads (v_readlane with a non-constant lane, v_movrel*).  Check a
+// new kernel's assembly for "m0" outside the s_mov_b32 of this statement.
 __device__ __forceinline__ void dtl_load(unsigned lds_dst, unsigned voff, const void* sbase) {
     asm volatile(
         "s_mov_b32 m0, %0\n\t"
@@ -140,6 +146,48 @@ struct DtlTile {
     }
 };
 
+// K split with the sum done in the kernel.  A product with few output tiles and a long K runs `splits` workgroups
+// per tile, workgroup (tile, s) summing K slice s.  After its K loop a workgroup draws a ticket from the tile's
+// counter.  All but the last to draw write their fp32 partial tile to the caller's workspace (in the accumulators'
+// own register order), report in on a second counter and are done; the last to draw waits until the others have
+// reported -- they drew before it, so they are past their K loops and their stores are in flight: a wait for
+// work already under way, never for a workgroup that may not have started -- adds the partials up in slice order
+// and runs the epilogue.  With more than two slices the last one writes its partial too and reads all of them
+// back in slice order, so the bits do not depend on which slice happened to draw last.
+// Partial tiles cross from one XCD's L2 to another's.  Every access to them is made coherent at device scope by
+// itself (the sc1 bit: the access goes to the level all XCDs share), so no fence has to write back or invalidate
+// a whole L2 -- which a device-scope fence does on this part, and which costs more than the product when a
+// thousand workgroups do it.
+// The counters live in the library, start at zero and are put back to zero by the last arrival, so a launch needs
+// no clearing pass; two products split at the same time on different streams of one device would share them and
+// must not overlap.
+constexpr int kMaxSplitTiles = 8192;
+static __device__ unsigned dtl_tickets[kMaxSplitTiles];
+static __device__ unsigned dtl_arrived[kMaxSplitTiles];
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+// The wait states after the store are part of the statement: a store of more than 64 bits reads its data
+// registers a few cycles after it issues, and the compiler, which keeps such a store's data registers intact for
+// that long when it emits the instruction itself, does not look into an asm statement -- it reused them for the
+// next address at once, and single lanes of a partial tile came out as garbage.
+__device__ __forceinline__ void store_device_coherent(f32x4* p, const f32x4& v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" : : "v"(p), "v"(v) : "memory");
+}
+// Four such loads and the wait for them in ONE statement: the compiler takes an asm statement's outputs to be
+// ready when the statement ends, so a wait in a statement of its own would let it copy the registers in between.
+__device__ __forceinline__ void load4_device_coherent(f32x4 (&v)[4], const f32x4* p, int stride) {
+    const f32x4 *p1 = p + stride, *p2 = p + 2 * stride, *p3 = p + 3 * stride;
+    asm volatile(
+        "global_load_dwordx4 %0, %4, off sc1\n\t"
+        "global_load_dwordx4 %1, %5, off sc1\n\t"
+        "global_load_dwordx4 %2, %6, off sc1\n\t"
+        "global_load_dwordx4 %3, %7, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3])
+        : "v"(p), "v"(p1), "v"(p2), "v"(p3)
+        : "memory");
+}
+
 template <int CT, int BM, int BN, int WM, int WN, int KT, int STAGES, bool A_KSTR, bool B_KSTR, typename TC,
           bool GELU = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(GemmArgs g) {
@@ -166,6 +214,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     tm = __builtin_amdgcn_readfirstlane(tm);
     tn = __builtin_amdgcn_readfirstlane(tn);
     batch = __builtin_amdgcn_readfirstlane((int)batch);
+    // with a K split the slices take the place of the batch index in the tile order (slice-major: the workgroups
+    // an XCD runs at a time still cover one block of tiles, of one slice)
+    const int slice = g.splits > 1 ? (int)batch : 0;
+    if (g.splits > 1) batch = 0;
     const long long row0 = (long long)tm * BM, col0 = (long long)tn * BN;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -194,11 +246,14 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
         for (int j = 0; j < FN; j++) fb_off[j][ks] = TA::kBytes + TB::frag_offset(wn * WN + j * 32, ks, lane);
     }
 
-    const int nk = (int)(g.k / KT);
-    // step `t` of the loop covers K step (t + first) mod nk (see k_walk_start)
-    const int first = (int)(k_walk_start(row0, col0, g.k) / KT);
-    a_src += first * a_step;
-    b_src += first * b_step;
+    // this workgroup's K steps: [k_begin, k_begin + nk) of the g.k / KT steps (all of them without a split)
+    const int nk_all = (int)(g.k / KT);
+    const int k_begin = (int)((long long)slice * nk_all / g.splits);
+    const int nk = (int)((long long)(slice + 1) * nk_all / g.splits) - k_begin;
+    // step `t` of the loop covers K step k_begin + (t + first) mod nk (see k_walk_start)
+    const int first = (int)(k_walk_start(row0, col0, g.k) / KT) % nk;
+    a_src += (k_begin + first) * a_step;
+    b_src += (k_begin + first) * b_step;
     int until_wrap = nk - first;  // issues left before the walk returns to K step 0
     auto issue = [&](int tile) {
         const unsigned dst = lds0 + (unsigned)(tile % STAGES) * kStageBytes + (unsigned)wave * 1024u;
@@ -290,6 +345,98 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                 __builtin_amdgcn_sched_barrier(0);
                 step(fa_now, fb_now, fa_next, fb_next, t + 1, 0);
             }
+        }
+    }
+
+    if (g.splits > 1) {
+        constexpr int THREADS = WAVES * 64;
+        constexpr size_t kTileQuads = (size_t)BM * BN / 4;
+        const int tile_id = tm * g.tiles_n + tn;
+        f32x4* const slots = reinterpret_cast<f32x4*>(g.partials) + (size_t)tile_id * g.splits * kTileQuads;
+        const bool two = g.splits == 2;
+        // everybody is through with the LDS tiles; one word of them carries the ticket to the workgroup
+        __syncthreads();
+        unsigned* const drawn = reinterpret_cast<unsigned*>(lds_raw);
+        if (threadIdx.x == 0)
+            *drawn = __hip_atomic_fetch_add(&dtl_tickets[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        const bool last = *drawn == (unsigned)g.splits - 1;
+        // Quad q of accumulator block (i, j) of thread t sits at quad index ((i*FN + j)*4 + q)*THREADS + t of a
+        // partial tile (a kilobyte per wave and instruction).  One block at a time, with a running pointer and a
+        // fence after each block: the kernel has no registers to spare for addresses formed ahead of time.
+        if (!(two && last)) {
+            f32x4* at = slots + (size_t)slice * kTileQuads + threadIdx.x;
+#pragma unroll
+            for (int blk = 0; blk < FM * FN; blk++) {
+                const int i = blk / FN, j = blk % FN;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    f32x4 v;
+                    v.x = acc[i][j][4 * q]; v.y = acc[i][j][4 * q + 1]; v.z = acc[i][j][4 * q + 2]; v.w = acc[i][j][4 * q + 3];
+                    store_device_coherent(at, v);
+                    at += THREADS;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            wait_vmem<0>();   // this thread's stores have reached the level every XCD sees
+        }
+        __syncthreads();      // ... and so have every other thread's of this workgroup
+        if (!last) {
+            if (threadIdx.x == 0) __hip_atomic_fetch_add(&dtl_arrived[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+        // The last to draw: the other slices drew before it, so each of them is past its K loop and on its way
+        // through the few lines above, which wait for nothing -- the wait below is for stores already in flight.
+        // The wait is bounded all the same (a second or so): should the counters ever be out of step -- a product
+        // killed half way leaves them so -- the tile is filled with NaN rather than summed from partials that are
+        // not there, and the kernel ends.
+        if (threadIdx.x == 0) {
+            unsigned seen = 0;
+            for (int spin = 0; spin < (1 << 22); spin++) {
+                seen = __hip_atomic_load(&dtl_arrived[tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (seen >= (unsigned)g.splits - 1) break;
+                __builtin_amdgcn_s_sleep(4);
+            }
+            *drawn = seen >= (unsigned)g.splits - 1 ? 1u : 0u;
+        }
+        __syncthreads();
+        if (*drawn == 0u) {
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[i][j][v] = __builtin_nanf("");
+        } else {
+        // Sum in slice order.  With two slices the sum is the same whichever term is the one held in registers, so
+        // only the other slice's partial exists and is read; with more, every slice is read back at its place in
+        // the order (this workgroup's own included), which makes the bits independent of which slice drew last.
+        for (int s = two ? (slice ^ 1) : 0; s < g.splits; s++) {
+            const f32x4* at = slots + (size_t)s * kTileQuads + threadIdx.x;
+            const bool adds = two || s > 0;
+#pragma unroll
+            for (int blk = 0; blk < FM * FN; blk++) {
+                const int i = blk / FN, j = blk % FN;
+                f32x4 v[4];
+                load4_device_coherent(v, at, THREADS);
+                at += 4 * THREADS;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    acc[i][j][4 * q] = adds ? acc[i][j][4 * q] + v[q].x : v[q].x;
+                    acc[i][j][4 * q + 1] = adds ? acc[i][j][4 * q + 1] + v[q].y : v[q].y;
+                    acc[i][j][4 * q + 2] = adds ? acc[i][j][4 * q + 2] + v[q].z : v[q].z;
+                    acc[i][j][4 * q + 3] = adds ? acc[i][j][4 * q + 3] + v[q].w : v[q].w;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (two) break;
+        }
+        }
+        if (threadIdx.x == 0) {
+            // ready for the next product; written the way the counters are read and added to (an ordinary store
+            // would sit in this XCD's L2, out of sight of the other XCDs' atomics, until the kernel ends)
+            __hip_atomic_store(&dtl_tickets[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&dtl_arrived[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 
@@ -397,7 +544,14 @@ int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t
     constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
     g.tiles_m = (int)((g.m + BM - 1) / BM);
     g.tiles_n = (int)((g.n + BN - 1) / BN);
-    const long long blocks = (long long)g.tiles_m * g.tiles_n * batch;
+    if (g.splits > 1) {
+        // the plan only splits unbatched products whose partial tiles fit the workspace it was given
+        const long long tiles = (long long)g.tiles_m * g.tiles_n;
+        if (batch != 1 || tiles > kMaxSplitTiles || !g.partials ||
+            (size_t)tiles * g.splits * BM * BN * sizeof(float) > g.partial_bytes)
+            return BR_ERR_ATTR;
+    }
+    const long long blocks = (long long)g.tiles_m * g.tiles_n * batch * g.splits;
     if (blocks > 0x7fffffffLL) return BR_ERR_ATTR;
     const unsigned grid = (unsigned)blocks;
     using F16 = __half;
@@ -440,37 +594,71 @@ inline bool dtl_applies(const GemmArgs& g, const Problem& p) {
     return a_span < lim && b_span < lim && g.ldc < (1LL << 27);
 }
 
-// Tile choice by estimated time: rounds of workgroups over the 256 CUs x the
-// MFMA work of one tile / the rate a workgroup of that configuration reaches
-// (measured on the BLOOM-7B1 linear-layer shapes: ~1000 TFLOP/s chip-wide for
-// 256x256, ~0.9 of that for 256x128, ~0.8 for 128x128 with two workgroups
-// resident per CU).
+// Tile and K-split choice by estimated time.  Per workgroup and 64-wide K step (MI355X, fp16, all CUs busy):
+// 1.8 us for a 256x256 tile, 1.15 us for 256x128, and for 128x128 0.8 us with the CU to itself and 1.16 us when two
+// such workgroups share it; 3 us per round of workgroups for filling and draining the pipeline; C leaves at
+// 6.5 TB/s.  A split adds its partial tiles: written by all slices but one (by all, when there are more than two)
+// and read back by one workgroup per tile, both through device-coherent accesses, which move 1.5-3 TB/s.
 struct DtlPlan {
     int config;      // 0: 256x256, 1: 256x128, 2: 128x128 (64-wide K steps), 3: 128x128 with 32-wide steps
+    int splits;      // workgroups per output tile (1 = K is not split)
     double seconds;  // estimate, for comparing plans only
 };
-inline DtlPlan dtl_plan(long long m, long long n, long long k, long long batch) {
-    const double per_cu = 1.0e15 / 256.0;  // flop/s of one CU at the 256x256 rate
-    auto estimate = [&](long long bm, long long bn, long long slots, double rel) {
+constexpr int kDtlTileM[4] = {256, 256, 128, 128}, kDtlTileN[4] = {256, 128, 128, 128};
+// bytes of partial tiles a plan needs in the caller's workspace
+inline size_t dtl_partial_bytes(const DtlPlan& p, long long m, long long n) {
+    if (p.splits <= 1) return 0;
+    const long long bm = kDtlTileM[p.config], bn = kDtlTileN[p.config];
+    return (size_t)(((m + bm - 1) / bm) * ((n + bn - 1) / bn)) * p.splits * bm * bn * sizeof(float);
+}
+// partial_budget: bytes available for partial tiles (0 = never split)
+inline DtlPlan dtl_plan(long long m, long long n, long long k, long long batch, size_t partial_budget = 0) {
+    auto estimate = [&](int config, int splits) {
+        const long long bm = kDtlTileM[config], bn = kDtlTileN[config];
         const long long tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch;
-        const double rounds = (double)((tiles + slots - 1) / slots);
-        const double per_block = per_cu * rel * 256.0 / (double)slots;  // co-resident workgroups share the CU
-        return rounds * 2.0 * (double)bm * (double)bn * (double)k / per_block + 4e-6;
+        const long long wgs = tiles * splits;
+        const long long slots = config >= 2 ? 512 : 256;
+        const double rounds = (double)((wgs + slots - 1) / slots);
+        const double steps = (double)(k / splits) / 64.0;
+        double step_us = config == 0 ? 1.8 : config == 1 ? 1.15 : (wgs > 256 ? 1.16 : 0.8);
+        if (config == 3) step_us *= 0.8 / 0.65;  // 32-wide K steps: two barriers where the others have one
+        double t = rounds * (steps * step_us + 3.0) * 1e-6 + (double)m * n * batch * 4.0 / 6.5e12 + 4e-6;
+        if (splits > 1) {
+            const double tile_bytes = (double)bm * bn * 4.0;
+            const double written = (double)tiles * (splits == 2 ? 1 : splits) * tile_bytes;
+            const double read = (double)tiles * (splits == 2 ? 1 : splits) * tile_bytes;
+            t += (written + read) / 3e12 + 3e-6;
+        }
+        return DtlPlan{config, splits, t};
     };
-    if (k % 64 != 0) return DtlPlan{3, estimate(128, 128, 512, 0.65)};
-    DtlPlan best{0, estimate(256, 256, 256, 1.0)};
-    const double t1 = estimate(256, 128, 256, 0.9), t2 = estimate(128, 128, 512, 0.8);
-    if (t1 < best.seconds) best = DtlPlan{1, t1};
-    if (t2 < best.seconds) best = DtlPlan{2, t2};
-    return best;
+    if (k % 64 != 0) return estimate(3, 1);
+    DtlPlan best = estimate(0, 1);
+    for (int c = 1; c < 3; c++) {
+        const DtlPlan p = estimate(c, 1);
+        if (p.seconds < best.seconds) best = p;
+    }
+    if (batch != 1 || partial_budget == 0) return best;
+    // a split has to win clearly: its partial tiles are traffic the unsplit product does not have
+    DtlPlan pick = best;
+    for (int c = 0; c < 3; c++)
+        for (int sp = 2; sp <= 8; sp *= 2) {
+            if (k / 64 / sp < 8) break;  // at least eight K steps per slice
+            const DtlPlan p = estimate(c, sp);
+            const long long bm = kDtlTileM[c], bn = kDtlTileN[c];
+            if (((m + bm - 1) / bm) * ((n + bn - 1) / bn) > kMaxSplitTiles) continue;
+            if (dtl_partial_bytes(p, m, n) > partial_budget) continue;
+            if (p.seconds < 0.97 * best.seconds && p.seconds < pick.seconds) pick = p;
+        }
+    return pick;
 }
 
 template <int CT>
-int launch_dtl(const GemmArgs& g, const Problem& p, long long batch, hipStream_t st) {
-    const int pick = dtl_plan(g.m, g.n, g.k, batch).config;
-    if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
-    if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
-    if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
+int launch_dtl(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
+    const DtlPlan plan = dtl_plan(g.m, g.n, g.k, batch, g.partials ? g.partial_bytes : 0);
+    g.splits = plan.splits;
+    if (plan.config == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
+    if (plan.config == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
+    if (plan.config == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
     return launch_dtl_config<CT, 128, 128, 64, 64, 32, 3>(g, p, batch, st);
 }
 
