@@ -378,16 +378,82 @@ int stage_rows(const float* src, long long ld, long long stride, long long rows,
 }
 
 // ---- split-K ------------------------------------------------------------------
-// A product with few output tiles and a long K leaves most CUs idle.  The
-// direct-to-LDS kernel can run several workgroups per tile, one per slice of K,
-// with the sum done by the workgroup that finishes last (gemm_dtl16.hpp); what
-// it needs from here is room for the partial tiles, after the staged operands.
-// The plan depends on the problem's sizes only, so a product's bits do not
-// depend on where its operands or its workspace happen to live.
-size_t split_room(int64_t m, int64_t n, int64_t k, int64_t batch) {
-    if (batch != 1 || k % 64 != 0) return 0;
-    const gemm16::DtlPlan plan = gemm16::dtl_plan(m, n, k, 1, ~(size_t)0);
-    return gemm16::dtl_partial_bytes(plan, m, n);
+// A product with few output tiles and a long K leaves most CUs idle.  Two forms,
+// both deterministic and free of floating-point atomics:
+//  * many slices (products with M = 512 or fewer rows: 4-16 slices): run as a
+//    strided-batched product over `splits` slices of K into fp32 partials (slice
+//    s of A / B is the operand advanced by s * k/splits along k, which the batch
+//    strides express), followed by a fixed-order sum in a second kernel;
+//  * two slices (M = 2048, N = 4096, K >= 12288: 128 tiles of 256 x 256 on 256
+//    CUs): inside the direct-to-LDS kernel, the slice that finishes last adds the
+//    other's partial tile and runs the epilogue (gemm_dtl16.hpp).  Measured on
+//    the same box, the in-kernel form loses to the two-kernel form when four or
+//    more slices exchange partial tiles (its device-coherent accesses move
+//    1.5-3 TB/s, ordinary stores 6-7) and wins with two, where only one of the
+//    two slices writes anything.
+// Which form, how many slices and which tile depend on the problem's sizes only,
+// so a product's bits do not depend on where its operands or its workspace
+// happen to live.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float4* __restrict__ part, int splits,
+                                                            long long mn4, long long n4, float alpha,
+                                                            const float* __restrict__ bias, const void* old,
+                                                            void* c, int c_dtype, long long ldc) {
+    for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < mn4;
+         i += (long long)gridDim.x * blockDim.x) {
+        float4 s = part[i];
+        for (int p = 1; p < splits; p++) {
+            const float4 v = part[(long long)p * mn4 + i];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        const long long row = i / n4, col = (i % n4) * 4;
+        float o[4] = {alpha * s.x, alpha * s.y, alpha * s.z, alpha * s.w};
+        if (bias) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) o[j] += bias[col + j];
+        }
+        if (c_dtype == BR_F32) {
+            // `old`: the tensor an accumulating product adds to (c itself or a tensor laid out like it), else null
+            float* dst = static_cast<float*>(c) + row * ldc + col;
+            const float* was = static_cast<const float*>(old) + row * ldc + col;
+#pragma unroll
+            for (int j = 0; j < 4; j++) dst[j] = old ? o[j] + was[j] : o[j];
+        } else if (c_dtype == BR_F16) {
+            __half* dst = static_cast<__half*>(c) + row * ldc + col;
+            const __half* was = static_cast<const __half*>(old) + row * ldc + col;
+#pragma unroll
+            for (int j = 0; j < 4; j++) dst[j] = __float2half_rn(old ? o[j] + __half2float(was[j]) : o[j]);
+        } else {
+            __hip_bfloat16* dst = static_cast<__hip_bfloat16*>(c) + row * ldc + col;
+            const __hip_bfloat16* was = static_cast<const __hip_bfloat16*>(old) + row * ldc + col;
+#pragma unroll
+            for (int j = 0; j < 4; j++) dst[j] = __float2bfloat16(old ? o[j] + __bfloat162float(was[j]) : o[j]);
+        }
+    }
+}
+
+// Number of K slices (1 = do not split) for an unbatched product on the
+// direct-to-LDS kernel: the split whose estimated time, including the pass
+// over the partials, is smallest.
+int splitk_choice(int64_t m, int64_t n, int64_t k) {
+    if (n % 4 != 0) return 1;
+    double best = gemm16::dtl_tile_plan(m, n, k, 1).seconds;
+    int pick = 1;
+    for (int s = 2; s <= 16; s *= 2) {
+        if (k % (64 * s) != 0 || k / s < 512) break;
+        const double t = gemm16::dtl_tile_plan(m, n, k / s, s).seconds + 6e-6 + (double)(s + 1) * m * n * 4.0 / 4e12;
+        if (t < 0.85 * best) {
+            best = t;
+            pick = s;
+        }
+    }
+    return pick;
+}
+
+
+// Bytes of partial tiles the two-slice in-kernel form wants (0 = it does not apply or does not pay).
+size_t pair_split_room(int64_t m, int64_t n, int64_t k, int64_t batch) {
+    if (batch != 1 || splitk_choice(m, n, k) > 1) return 0;
+    return gemm16::dtl_pair_split_bytes(m, n, k);
 }
 
 size_t staged_bytes(int64_t rows, int64_t cols, int64_t batch) {
@@ -405,7 +471,11 @@ extern "C" size_t br_hip_gemm_staged_workspace(int trans_a, int trans_b, int64_t
     size_t need = 0;
     if (a_dtype == BR_F32) need += staged_bytes(m, k, batch);
     if (b_dtype == BR_F32) need += staged_bytes(k, n, batch);
-    need += split_room(m, n, k, batch);
+    if (batch == 1) {
+        const int splits = splitk_choice(m, n, k);
+        if (splits > 1) need += (size_t)splits * (size_t)m * (size_t)n * sizeof(float);
+    }
+    need += pair_split_room(m, n, k, batch);
     return need;
 }
 
@@ -456,9 +526,27 @@ int staged_impl(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float
         stride_b = b_rows * b_cols;
         ws += staged_bytes(k, n, batch);
     }
-    // what is left of the workspace holds the partial tiles of a K split; the plan is made for the room the
-    // workspace function asked for and the product is split only if that much is really there
-    const size_t room = split_room(m, n, k, batch);
+    const int splits = batch == 1 ? splitk_choice(m, n, k) : 1;
+    if (splits > 1 && c) {
+        // slices of K as batch entries: a k-contiguous operand advances by k/splits
+        // elements per slice, a row-contiguous one by k/splits rows
+        const int64_t ks = k / splits;
+        float* part = reinterpret_cast<float*>(ws);
+        const int rc = br_hip_gemm(trans_a, trans_b, m, n, ks, 1.0f, a, a_dtype, lda, trans_a ? ks * lda : ks, b,
+                                   b_dtype, ldb, trans_b ? ks : ks * ldb, 0, part, BR_F32, n, m * n, nullptr, splits,
+                                   compute, stream);
+        if (rc != BR_OK) return rc;
+        const long long mn4 = m * n / 4;
+        splitk_reduce_kernel<<<grid_for(mn4, 256, 1 << 14), 256, 0, st>>>(reinterpret_cast<const float4*>(part),
+                                                                        splits, mn4, n / 4, alpha, bias,
+                                                                        accumulate ? (addend ? addend : c) : nullptr,
+                                                                        c, c_dtype, ldc);
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
+    }
+    // two slices inside the kernel: what is left of the workspace holds one partial tile per output tile; the
+    // product is split only if the room the workspace function asked for is really there
+    const size_t room = pair_split_room(m, n, k, batch);
     const size_t left = workspace_bytes - (size_t)(ws - static_cast<char*>(workspace));
     float* partials = room > 0 && room <= left ? reinterpret_cast<float*>(ws) : nullptr;
     return gemm_impl(trans_a, trans_b, m, n, k, alpha, a, a_dtype, lda, stride_a, b, b_dtype, ldb, stride_b, accumulate,

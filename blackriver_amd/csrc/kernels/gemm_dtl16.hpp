@@ -146,19 +146,21 @@ struct DtlTile {
     }
 };
 
-// K split with the sum done in the kernel.  A product with few output tiles and a long K runs `splits` workgroups
-// per tile, workgroup (tile, s) summing K slice s.  After its K loop a workgroup draws a ticket from the tile's
-// counter.  All but the last to draw write their fp32 partial tile to the caller's workspace (in the accumulators'
-// own register order), report in on a second counter and are done; the last to draw waits until the others have
-// reported -- they drew before it, so they are past their K loops and their stores are in flight: a wait for
-// work already under way, never for a workgroup that may not have started -- adds the partials up in slice order
-// and runs the epilogue.  With more than two slices the last one writes its partial too and reads all of them
-// back in slice order, so the bits do not depend on which slice happened to draw last.
-// Partial tiles cross from one XCD's L2 to another's.  Every access to them is made coherent at device scope by
+// K split in two with the sum done in the kernel.  A product whose 256x256 tiles fill at most half the CUs and
+// whose K is long runs two workgroups per tile, workgroup (tile, s) summing half s of K.  After its K loop a
+// workgroup draws a ticket from the tile's counter.  The first to draw writes its fp32 partial tile to the caller's
+// workspace (in the accumulators' own register order), reports in on a second counter and is done; the second
+// waits until the first has reported -- it drew first, so it is past its K loop and its stores are in flight: a
+// wait for work already under way, never for a workgroup that may not have started -- adds that partial to its own
+// and runs the epilogue.  A sum of two terms is the same whichever is added to which, so the bits do not depend on
+// which half finished first.
+// The partial tile crosses from one XCD's L2 to another's.  Every access to it is made coherent at device scope by
 // itself (the sc1 bit: the access goes to the level all XCDs share), so no fence has to write back or invalidate
-// a whole L2 -- which a device-scope fence does on this part, and which costs more than the product when a
-// thousand workgroups do it.
-// The counters live in the library, start at zero and are put back to zero by the last arrival, so a launch needs
+// a whole L2 -- which a device-scope fence does on this part, and which costs more than the product when hundreds
+// of workgroups do it.  Such accesses move 1.5-3 TB/s where ordinary stores move 6-7: with four or more slices
+// (every slice writing, one reading them all) this form measured slower than partials written with ordinary
+// stores and summed by a second kernel, which is what products with more slices use (gemm.hip).
+// The counters live in the library, start at zero and are put back to zero by the second arrival, so a launch needs
 // no clearing pass; two products split at the same time on different streams of one device would share them and
 // must not overlap.
 constexpr int kMaxSplitTiles = 8192;
@@ -189,7 +191,7 @@ __device__ __forceinline__ void load4_device_coherent(f32x4 (&v)[4], const f32x4
 }
 
 template <int CT, int BM, int BN, int WM, int WN, int KT, int STAGES, bool A_KSTR, bool B_KSTR, typename TC,
-          bool GELU = false>
+          bool GELU = false, bool SPLIT = false>
 __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(GemmArgs g) {
     constexpr int WAVES = (BM / WM) * (BN / WN);
     constexpr int FM = WM / 32, FN = WN / 32, KS = KT / 16;
@@ -216,8 +218,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     batch = __builtin_amdgcn_readfirstlane((int)batch);
     // with a K split the slices take the place of the batch index in the tile order (slice-major: the workgroups
     // an XCD runs at a time still cover one block of tiles, of one slice)
-    const int slice = g.splits > 1 ? (int)batch : 0;
-    if (g.splits > 1) batch = 0;
+    const int slice = SPLIT ? (int)batch : 0;
+    if (SPLIT) batch = 0;
     const long long row0 = (long long)tm * BM, col0 = (long long)tn * BN;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -248,10 +250,10 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
 
     // this workgroup's K steps: [k_begin, k_begin + nk) of the g.k / KT steps (all of them without a split)
     const int nk_all = (int)(g.k / KT);
-    const int k_begin = (int)((long long)slice * nk_all / g.splits);
-    const int nk = (int)((long long)(slice + 1) * nk_all / g.splits) - k_begin;
+    const int k_begin = SPLIT ? slice * nk_all / 2 : 0;
+    const int nk = SPLIT ? (slice + 1) * nk_all / 2 - k_begin : nk_all;
     // step `t` of the loop covers K step k_begin + (t + first) mod nk (see k_walk_start)
-    const int first = (int)(k_walk_start(row0, col0, g.k) / KT) % nk;
+    const int first = SPLIT ? (int)(k_walk_start(row0, col0, g.k) / KT) % nk : (int)(k_walk_start(row0, col0, g.k) / KT);
     a_src += (k_begin + first) * a_step;
     b_src += (k_begin + first) * b_step;
     int until_wrap = nk - first;  // issues left before the walk returns to K step 0
@@ -348,24 +350,23 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
         }
     }
 
-    if (g.splits > 1) {
+    if constexpr (SPLIT) {
         constexpr int THREADS = WAVES * 64;
         constexpr size_t kTileQuads = (size_t)BM * BN / 4;
         const int tile_id = tm * g.tiles_n + tn;
-        f32x4* const slots = reinterpret_cast<f32x4*>(g.partials) + (size_t)tile_id * g.splits * kTileQuads;
-        const bool two = g.splits == 2;
+        f32x4* const slot = reinterpret_cast<f32x4*>(g.partials) + (size_t)tile_id * kTileQuads;
         // everybody is through with the LDS tiles; one word of them carries the ticket to the workgroup
         __syncthreads();
         unsigned* const drawn = reinterpret_cast<unsigned*>(lds_raw);
         if (threadIdx.x == 0)
             *drawn = __hip_atomic_fetch_add(&dtl_tickets[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
-        const bool last = *drawn == (unsigned)g.splits - 1;
-        // Quad q of accumulator block (i, j) of thread t sits at quad index ((i*FN + j)*4 + q)*THREADS + t of a
+        const bool last = *drawn == 1u;
+        // Quad q of accumulator block (i, j) of thread t sits at quad index ((i*FN + j)*4 + q)*THREADS + t of the
         // partial tile (a kilobyte per wave and instruction).  One block at a time, with a running pointer and a
         // fence after each block: the kernel has no registers to spare for addresses formed ahead of time.
-        if (!(two && last)) {
-            f32x4* at = slots + (size_t)slice * kTileQuads + threadIdx.x;
+        if (!last) {
+            f32x4* at = slot + threadIdx.x;
 #pragma unroll
             for (int blk = 0; blk < FM * FN; blk++) {
                 const int i = blk / FN, j = blk % FN;
@@ -379,25 +380,23 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                 __builtin_amdgcn_sched_barrier(0);
             }
             wait_vmem<0>();   // this thread's stores have reached the level every XCD sees
-        }
-        __syncthreads();      // ... and so have every other thread's of this workgroup
-        if (!last) {
-            if (threadIdx.x == 0) __hip_atomic_fetch_add(&dtl_arrived[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __syncthreads();  // ... and so have every other thread's of this workgroup
+            if (threadIdx.x == 0)
+                __hip_atomic_fetch_add(&dtl_arrived[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             return;
         }
-        // The last to draw: the other slices drew before it, so each of them is past its K loop and on its way
-        // through the few lines above, which wait for nothing -- the wait below is for stores already in flight.
-        // The wait is bounded all the same (a second or so): should the counters ever be out of step -- a product
-        // killed half way leaves them so -- the tile is filled with NaN rather than summed from partials that are
-        // not there, and the kernel ends.
+        // The second to draw: the other slice drew first, so it is past its K loop and on its way through the few
+        // lines above, which wait for nothing -- the wait below is for stores already in flight.  It is bounded all
+        // the same (a second or so): should the counters ever be out of step -- a product killed half way leaves
+        // them so -- the tile is filled with NaN rather than summed from a partial that is not there.
         if (threadIdx.x == 0) {
             unsigned seen = 0;
             for (int spin = 0; spin < (1 << 22); spin++) {
                 seen = __hip_atomic_load(&dtl_arrived[tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (seen >= (unsigned)g.splits - 1) break;
+                if (seen >= 1u) break;
                 __builtin_amdgcn_s_sleep(4);
             }
-            *drawn = seen >= (unsigned)g.splits - 1 ? 1u : 0u;
+            *drawn = seen >= 1u ? 1u : 0u;
         }
         __syncthreads();
         if (*drawn == 0u) {
@@ -408,12 +407,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
 #pragma unroll
                     for (int v = 0; v < 16; v++) acc[i][j][v] = __builtin_nanf("");
         } else {
-        // Sum in slice order.  With two slices the sum is the same whichever term is the one held in registers, so
-        // only the other slice's partial exists and is read; with more, every slice is read back at its place in
-        // the order (this workgroup's own included), which makes the bits independent of which slice drew last.
-        for (int s = two ? (slice ^ 1) : 0; s < g.splits; s++) {
-            const f32x4* at = slots + (size_t)s * kTileQuads + threadIdx.x;
-            const bool adds = two || s > 0;
+            // two terms: the sum is the same whichever of them is the one held in registers, so the bits do not
+            // depend on which slice drew last
+            const f32x4* at = slot + threadIdx.x;
 #pragma unroll
             for (int blk = 0; blk < FM * FN; blk++) {
                 const int i = blk / FN, j = blk % FN;
@@ -422,15 +418,13 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                 at += 4 * THREADS;
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    acc[i][j][4 * q] = adds ? acc[i][j][4 * q] + v[q].x : v[q].x;
-                    acc[i][j][4 * q + 1] = adds ? acc[i][j][4 * q + 1] + v[q].y : v[q].y;
-                    acc[i][j][4 * q + 2] = adds ? acc[i][j][4 * q + 2] + v[q].z : v[q].z;
-                    acc[i][j][4 * q + 3] = adds ? acc[i][j][4 * q + 3] + v[q].w : v[q].w;
+                    acc[i][j][4 * q] += v[q].x;
+                    acc[i][j][4 * q + 1] += v[q].y;
+                    acc[i][j][4 * q + 2] += v[q].z;
+                    acc[i][j][4 * q + 3] += v[q].w;
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (two) break;
-        }
         }
         if (threadIdx.x == 0) {
             // ready for the next product; written the way the counters are read and added to (an ordinary store
@@ -547,8 +541,8 @@ int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t
     if (g.splits > 1) {
         // the plan only splits unbatched products whose partial tiles fit the workspace it was given
         const long long tiles = (long long)g.tiles_m * g.tiles_n;
-        if (batch != 1 || tiles > kMaxSplitTiles || !g.partials ||
-            (size_t)tiles * g.splits * BM * BN * sizeof(float) > g.partial_bytes)
+        if (g.splits != 2 || batch != 1 || tiles > kMaxSplitTiles || !g.partials ||
+            (size_t)tiles * BM * BN * sizeof(float) > g.partial_bytes)   // one partial tile per output tile
             return BR_ERR_ATTR;
     }
     const long long blocks = (long long)g.tiles_m * g.tiles_n * batch * g.splits;
@@ -556,6 +550,27 @@ int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t
     const unsigned grid = (unsigned)blocks;
     using F16 = __half;
     using BF16 = __hip_bfloat16;
+    if (g.splits == 2) {
+        // the two-slice form: its own instantiations (of the two 256-row tiles, the only ones it is planned on),
+        // so that the unsplit kernels carry none of its code
+        if (g.c2 || BM != 256) return BR_ERR_TODO;
+#define BR_DTL_SPLIT_CASE(AK, BK_)                                                                              \
+    if constexpr (BM == 256) if (p.a_kstr == AK && p.b_kstr == BK_) {                                                                     \
+        if (p.c_dtype == BR_F32)                                                                                 \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, float, false, true><<<grid, THREADS, 0, st>>>(g); \
+        else if (CT == BR_GEMM_F16)                                                                              \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, F16, false, true><<<grid, THREADS, 0, st>>>(g);   \
+        else                                                                                                     \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, BF16, false, true><<<grid, THREADS, 0, st>>>(g);  \
+    }
+        BR_DTL_SPLIT_CASE(false, false)
+        BR_DTL_SPLIT_CASE(false, true)
+        BR_DTL_SPLIT_CASE(true, false)
+        BR_DTL_SPLIT_CASE(true, true)
+#undef BR_DTL_SPLIT_CASE
+        BR_HIP_LAUNCH_CHECK();
+        return BR_OK;
+    }
     if (g.c2) {
         // GELU epilogue: built for the linear layer's layout only (both operands k-contiguous, 16-bit outputs)
         if (p.a_kstr || p.b_kstr || p.c_dtype == BR_F32) return BR_ERR_TODO;
@@ -594,71 +609,86 @@ inline bool dtl_applies(const GemmArgs& g, const Problem& p) {
     return a_span < lim && b_span < lim && g.ldc < (1LL << 27);
 }
 
-// Tile and K-split choice by estimated time.  Per workgroup and 64-wide K step (MI355X, fp16, all CUs busy):
-// 1.8 us for a 256x256 tile, 1.15 us for 256x128, and for 128x128 0.8 us with the CU to itself and 1.16 us when two
-// such workgroups share it; 3 us per round of workgroups for filling and draining the pipeline; C leaves at
-// 6.5 TB/s.  A split adds its partial tiles: written by all slices but one (by all, when there are more than two)
-// and read back by one workgroup per tile, both through device-coherent accesses, which move 1.5-3 TB/s.
+// Tile choice by estimated time: rounds of workgroups over the 256 CUs x the
+// MFMA work of one tile / the rate a workgroup of that configuration reaches
+// (measured on the BLOOM-7B1 linear-layer shapes: ~1000 TFLOP/s chip-wide for
+// 256x256, ~0.9 of that for 256x128, ~0.8 for 128x128 with two workgroups
+// resident per CU).
 struct DtlPlan {
     int config;      // 0: 256x256, 1: 256x128, 2: 128x128 (64-wide K steps), 3: 128x128 with 32-wide steps
-    int splits;      // workgroups per output tile (1 = K is not split)
     double seconds;  // estimate, for comparing plans only
 };
-constexpr int kDtlTileM[4] = {256, 256, 128, 128}, kDtlTileN[4] = {256, 128, 128, 128};
-// bytes of partial tiles a plan needs in the caller's workspace
-inline size_t dtl_partial_bytes(const DtlPlan& p, long long m, long long n) {
-    if (p.splits <= 1) return 0;
-    const long long bm = kDtlTileM[p.config], bn = kDtlTileN[p.config];
-    return (size_t)(((m + bm - 1) / bm) * ((n + bn - 1) / bn)) * p.splits * bm * bn * sizeof(float);
-}
-// partial_budget: bytes available for partial tiles (0 = never split)
-inline DtlPlan dtl_plan(long long m, long long n, long long k, long long batch, size_t partial_budget = 0) {
-    auto estimate = [&](int config, int splits) {
-        const long long bm = kDtlTileM[config], bn = kDtlTileN[config];
+inline DtlPlan dtl_tile_plan(long long m, long long n, long long k, long long batch) {
+    const double per_cu = 1.0e15 / 256.0;  // flop/s of one CU at the 256x256 rate
+    auto estimate = [&](long long bm, long long bn, long long slots, double rel) {
         const long long tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch;
-        const long long wgs = tiles * splits;
-        const long long slots = config >= 2 ? 512 : 256;
-        const double rounds = (double)((wgs + slots - 1) / slots);
-        const double steps = (double)(k / splits) / 64.0;
-        double step_us = config == 0 ? 1.8 : config == 1 ? 1.15 : (wgs > 256 ? 1.16 : 0.8);
-        if (config == 3) step_us *= 0.8 / 0.65;  // 32-wide K steps: two barriers where the others have one
-        double t = rounds * (steps * step_us + 3.0) * 1e-6 + (double)m * n * batch * 4.0 / 6.5e12 + 4e-6;
-        if (splits > 1) {
-            const double tile_bytes = (double)bm * bn * 4.0;
-            const double written = (double)tiles * (splits == 2 ? 1 : splits) * tile_bytes;
-            const double read = (double)tiles * (splits == 2 ? 1 : splits) * tile_bytes;
-            t += (written + read) / 3e12 + 3e-6;
-        }
-        return DtlPlan{config, splits, t};
+        const double rounds = (double)((tiles + slots - 1) / slots);
+        const double per_block = per_cu * rel * 256.0 / (double)slots;  // co-resident workgroups share the CU
+        return rounds * 2.0 * (double)bm * (double)bn * (double)k / per_block + 4e-6;
     };
-    if (k % 64 != 0) return estimate(3, 1);
-    DtlPlan best = estimate(0, 1);
-    for (int c = 1; c < 3; c++) {
-        const DtlPlan p = estimate(c, 1);
-        if (p.seconds < best.seconds) best = p;
-    }
-    if (batch != 1 || partial_budget == 0) return best;
-    // a split has to win clearly: its partial tiles are traffic the unsplit product does not have
-    DtlPlan pick = best;
-    for (int c = 0; c < 3; c++)
-        for (int sp = 2; sp <= 8; sp *= 2) {
-            if (k / 64 / sp < 8) break;  // at least eight K steps per slice
-            const DtlPlan p = estimate(c, sp);
-            const long long bm = kDtlTileM[c], bn = kDtlTileN[c];
-            if (((m + bm - 1) / bm) * ((n + bn - 1) / bn) > kMaxSplitTiles) continue;
-            if (dtl_partial_bytes(p, m, n) > partial_budget) continue;
-            if (p.seconds < 0.97 * best.seconds && p.seconds < pick.seconds) pick = p;
+    if (k % 64 != 0) return DtlPlan{3, estimate(128, 128, 512, 0.65)};
+    DtlPlan best{0, estimate(256, 256, 256, 1.0)};
+    const double t1 = estimate(256, 128, 256, 0.9), t2 = estimate(128, 128, 512, 0.8);
+    if (t1 < best.seconds) best = DtlPlan{1, t1};
+    if (t2 < best.seconds) best = DtlPlan{2, t2};
+    return best;
+}
+
+// Whether the two-slice K split inside the kernel pays (-1 = no, else the tile configuration to run it with), from
+// per-workgroup times measured on MI355X (fp16, all CUs busy): a 64-wide K step takes 1.8 us on a 256x256 tile and
+// 1.15 us on 256x128; a round of workgroups costs 3 us to fill and drain; C leaves at 6.5 TB/s; the one partial tile
+// per output tile is written and read back through device-coherent accesses at about 3 TB/s.  It pays where 256x256
+// tiles would fill at most half the CUs and K is long: for [2048 x 4096] outputs from K = 12288 up (8-10 % there).
+// Shorter M (few rows: many slices do better, see the caller) and shapes this timing was not taken on are left alone.
+inline int dtl_pair_split(long long m, long long n, long long k) {
+    if (m < 1024 || k % 64 != 0 || k / 64 < 16) return -1;
+    auto estimate = [&](int config, int splits) {
+        const long long bm = config == 0 ? 256 : 256, bn = config == 0 ? 256 : 128;
+        const long long tiles = ((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+        const double rounds = (double)((tiles * splits + 255) / 256);
+        const double steps = (double)(k / splits) / 64.0;
+        double t = rounds * (steps * (config == 0 ? 1.8 : 1.15) + 3.0) * 1e-6 + (double)m * n * 4.0 / 6.5e12 + 4e-6;
+        if (splits > 1) t += 2.0 * (double)tiles * bm * bn * 4.0 / 3e12 + 3e-6;
+        return t;
+    };
+    const double unsplit = estimate(0, 1) < estimate(1, 1) ? estimate(0, 1) : estimate(1, 1);
+    int pick = -1;
+    double best = 0.97 * unsplit;
+    for (int c = 0; c < 2; c++) {
+        const long long bm = 256, bn = c == 0 ? 256 : 128;
+        if (((m + bm - 1) / bm) * ((n + bn - 1) / bn) > kMaxSplitTiles) continue;
+        const double t = estimate(c, 2);
+        if (t < best) {
+            best = t;
+            pick = c;
         }
+    }
     return pick;
+}
+// bytes of partial tiles the two-slice split needs in the caller's workspace (one per output tile; 0 when the
+// split does not pay)
+inline size_t dtl_pair_split_bytes(long long m, long long n, long long k) {
+    const int c = dtl_pair_split(m, n, k);
+    if (c < 0) return 0;
+    const long long bm = 256, bn = c == 0 ? 256 : 128;
+    return (size_t)(((m + bm - 1) / bm) * ((n + bn - 1) / bn)) * bm * bn * sizeof(float);
 }
 
 template <int CT>
 int launch_dtl(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
-    const DtlPlan plan = dtl_plan(g.m, g.n, g.k, batch, g.partials ? g.partial_bytes : 0);
-    g.splits = plan.splits;
-    if (plan.config == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
-    if (plan.config == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
-    if (plan.config == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
+    g.splits = 1;
+    if (batch == 1 && g.partials) {
+        const int c = dtl_pair_split(g.m, g.n, g.k);
+        if (c >= 0 && dtl_pair_split_bytes(g.m, g.n, g.k) <= g.partial_bytes) {
+            g.splits = 2;
+            if (c == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
+            return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
+        }
+    }
+    const int pick = dtl_tile_plan(g.m, g.n, g.k, batch).config;
+    if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
+    if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
+    if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
     return launch_dtl_config<CT, 128, 128, 64, 64, 32, 3>(g, p, batch, st);
 }
 

@@ -70,9 +70,9 @@ struct GemmArgs {
     // what an accumulating product adds to: a tensor laid out like c (same type, leading dimension and batch
     // stride), read where c is written; null = c itself
     const void* addend = nullptr;
-    // K split of the direct-to-LDS kernel: `splits` workgroups share an output tile, each summing one slice of K;
-    // they leave their fp32 partial tiles in `partials` and the one that finishes last adds them up and runs the
-    // epilogue (see gemm_dtl16.hpp).  splits == 1: no split, partials unused.
+    // K split of the direct-to-LDS kernel: with splits == 2 two workgroups share an output tile, each summing one
+    // half of K; the first to finish leaves its fp32 partial tile in `partials`, the second adds it to its own and
+    // runs the epilogue (see gemm_dtl16.hpp).  splits == 1: no split, partials unused.
     int splits = 1;
     float* partials = nullptr;
     size_t partial_bytes = 0;
