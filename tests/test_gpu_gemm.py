@@ -194,6 +194,26 @@ def test_gemm_direct_to_lds_at_linear_layer_shape():
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("n,c_dt", [(12288, F16), (12248, F32)])
+def test_gemm_round_and_a_half_of_tiles(ta, tb, n, c_dt):
+    """[2048 x 12288] from K = 1024: 384 tiles of 256 x 256 are a round and a
+    half on 256 CUs, which the dispatcher runs as two launches (8192 columns on
+    256 x 256 tiles, the rest on 256 x 128 tiles).  Bias, alpha and an
+    accumulated C cross the seam; the ragged case ends inside the second
+    launch's last tile."""
+    rng = np.random.default_rng(21)
+    m, k = 2048, 1024
+    print("case ta=%d tb=%d n=%d c_dt=%d" % (ta, tb, n, c_dt), flush=True)
+    a, b = operands(rng, ta, tb, m, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c0 = rng.standard_normal((1, m, n)).astype(np.float32)
+    got, ref = run_gemm(ta, tb, m, n, k, a, b, F16, F16, c_dt, hip.GEMM_F16, alpha=0.5, bias=bias, c0=c0)
+    assert_close(got, ref, 2e-2, "two-launch product")
+    if c_dt == F32:
+        assert np.sqrt(np.mean((got - ref) ** 2)) < 1e-5 * np.sqrt(np.mean(ref ** 2)) * np.sqrt(k)
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
 @pytest.mark.parametrize("a_dt,b_dt", [(F32, F16), (F16, F32), (F32, F32)])
 def test_gemm_staged_matches_plain_entry(ta, tb, a_dt, b_dt):
     rng = np.random.default_rng(8)
@@ -262,7 +282,7 @@ def test_gemm_rejects_bad_arguments():
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("rows,out,inn", [(512, 1024, 256), (200, 520, 96), (2048, 4096, 1024)])
+@pytest.mark.parametrize("rows,out,inn", [(512, 1024, 256), (200, 520, 96), (2048, 4096, 1024), (2048, 12288, 1024)])
 def test_linear_gelu_epilogue_writes_both_tensors(dtype, rows, out, inn):
     """br_hip_linear_gelu: u = x.W^T + bias and y = gelu(u) from one product.
     u against the fp64 product of the stored operands, y against the oracle's
