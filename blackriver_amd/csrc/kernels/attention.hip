@@ -351,32 +351,6 @@ __device__ __forceinline__ float to_f32<BR_GEMM_F16>(u16 x) { return (float)__bu
 template <>
 __device__ __forceinline__ float to_f32<BR_GEMM_BF16>(u16 x) { return __uint_as_float((unsigned)x << 16); }
 
-// delta[b, h, t] = sum_d dO[b, t, h, d] * O[b, t, h, d]: 16 lanes per row.
-template <int CT>
-__global__ __launch_bounds__(kThreads) void flash_delta_kernel(FlashArgs a, long long rows) {
-    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
-    long long r = idx >> 4;
-    const bool live = r < rows;
-    r = live ? r : rows - 1;
-    const int part = (int)(idx & 15);
-    const int h = (int)(r % a.heads);
-    const long long bt = r / a.heads;
-    const int t = (int)(bt % a.tokens);
-    const long long b = bt / a.tokens;
-    const long long off = b * a.obatch + (long long)t * a.orow + (long long)h * a.head + part * 8;
-    const u32x4 g = *reinterpret_cast<const u32x4*>(a.d_o + off);
-    const u32x4 y = *reinterpret_cast<const u32x4*>(a.o + off);
-    float sum = 0.f;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        sum += to_f32<CT>((u16)(g[j] & 0xffffu)) * to_f32<CT>((u16)(y[j] & 0xffffu));
-        sum += to_f32<CT>((u16)(g[j] >> 16)) * to_f32<CT>((u16)(y[j] >> 16));
-    }
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, kWave);
-    if (live && part == 0) a.delta[(b * a.heads + h) * a.tokens + t] = sum;
-}
-
 // One LDS stage of the query loop of the dK / dV pass: a Q tile, a dO tile and
 // the tile's lse and delta values.
 constexpr int kQStageBytes = 2 * kTileBytes + 2 * kBK * 4;
@@ -568,16 +542,29 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
     const int qrow = query < a.tokens ? query : a.tokens - 1;
     const float* alibi_row = a.alibi + (long long)h * a.tokens;
     const float lse = a.lse[(long long)bh * a.tokens + qrow];
-    const float delta = a.delta[(long long)bh * a.tokens + qrow];
     const float uniform = 1.0f / (float)a.tokens;
 
+    // The query's dO fragments, and on the way delta[query] = sum_d dO[query, d] * O[query, d]: the two halves of a
+    // wave hold the two halves of every 16-wide slice of the row.  The dK / dV pass, which runs after this one,
+    // reads the value from a.delta.
     u32x4 qf[8], gf[8];
+    const long long orow = (long long)b * a.obatch + (long long)h * a.head + (long long)qrow * a.orow;
+    float delta = 0.f;
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) {
-        qf[ks] = *reinterpret_cast<const u32x4*>(a.q + base + (long long)qrow * a.row + ks * 16 + half * 8);
-        gf[ks] = *reinterpret_cast<const u32x4*>(a.d_o + (long long)b * a.obatch + (long long)h * a.head +
-                                                 (long long)qrow * a.orow + ks * 16 + half * 8);
+        gf[ks] = *reinterpret_cast<const u32x4*>(a.d_o + orow + ks * 16 + half * 8);
+        const u32x4 y = *reinterpret_cast<const u32x4*>(a.o + orow + ks * 16 + half * 8);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            delta += to_f32<CT>((u16)(gf[ks][j] & 0xffffu)) * to_f32<CT>((u16)(y[j] & 0xffffu));
+            delta += to_f32<CT>((u16)(gf[ks][j] >> 16)) * to_f32<CT>((u16)(y[j] >> 16));
+        }
     }
+    delta += __shfl_xor(delta, 32, kWave);
+    if (half == 0 && query < a.tokens) a.delta[(long long)bh * a.tokens + query] = delta;
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++)
+        qf[ks] = *reinterpret_cast<const u32x4*>(a.q + base + (long long)qrow * a.row + ks * 16 + half * 8);
     f32x16 dq[4];
 #pragma unroll
     for (int db = 0; db < 4; db++)
@@ -744,6 +731,9 @@ int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     if (batch == 0) return BR_OK;
     if (!q || !k || !v || !o || !d_o || !alibi || !valid || !lse) return BR_ERR_INPUT;
     if (!delta || !dq || !dk || !dv) return BR_ERR_OUTPUT;
+    for (const void* out : {(const void*)dq, (const void*)dk, (const void*)dv})
+        for (const void* in : {q, k, v, o, d_o})
+            if (out == in) return BR_ERR_OUTPUT;   // both passes read every input
     if (grad_dtype != BR_F32 && grad_dtype != dtype) return BR_ERR_TODO;
     if ((dtype != BR_F16 && dtype != BR_BF16) ||
         !flash_shape_ok(batch, heads, tokens, head_dim, row_stride, head_stride, batch_stride, o_row_stride,
@@ -775,17 +765,14 @@ int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     a.batch_heads = (int)(batch * heads);
     a.scale = (float)(1.0 / sqrt((double)head_dim));
     hipStream_t st = as_stream(stream);
-    const long long rows = batch * tokens * heads;
     const unsigned tiles = (unsigned)(((tokens + kBQ - 1) / kBQ) * batch * heads);
-    const unsigned dgrid = (unsigned)((rows * 16 + kThreads - 1) / kThreads);
+    // the dQ pass first: it leaves delta behind for the dK / dV pass
     if (dtype == BR_F16) {
-        flash_delta_kernel<BR_GEMM_F16><<<dgrid, kThreads, 0, st>>>(a, rows);
-        flash_bwd_dkv_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
         flash_bwd_dq_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
+        flash_bwd_dkv_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
     } else {
-        flash_delta_kernel<BR_GEMM_BF16><<<dgrid, kThreads, 0, st>>>(a, rows);
-        flash_bwd_dkv_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
         flash_bwd_dq_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
+        flash_bwd_dkv_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
     }
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;

@@ -646,6 +646,168 @@ int colsum_vec_rows_per_block(int64_t rows, int64_t blocks_x) {
     return (int)rpb;
 }
 
+// ------------------------------------------------ column sums in one launch
+// A workgroup of 1024 threads owns 8 * VEC columns (128 bytes of a 16-bit row, 128 bytes of an fp32 row) and walks
+// ALL rows: 8 lanes per row, 128 rows per pass, UNROLL passes in flight.  No partial sums leave the workgroup and
+// there is no second launch; the 128 row slots are combined in LDS in a fixed order, so the result depends on the
+// shape alone.  Measured against the two launches: 16-bit [2048,12288] 11.4 against 15.5 us, [2048,16384] 14.3
+// against 18.9, [512,16384] 4.6 against 11.0; fp32 [512,4096] with a 16-bit copy 3.9 against 6.6 -- but fp32
+// [2048,4096] 17 against 13.4 (128 workgroups are too few for 50 MB) and the fp16 bias-GELU backward at [2048,16384]
+// 44.5 against 43.0 (its arithmetic wants more waves than 1024 threads per CU give), which therefore keep the two
+// launches above 1024 rows (colsum_owner_applies).  Whole BLOOM-7B1 step at 512 tokens: -0.9 %.  What is summed, and what else is written on the way, is the Source's business:
+//   load(at, in)      the loads of one row position (all of a pass's loads are issued before any is used)
+//   finish(at, in)    leaves the values to be summed in in[0]; may store
+template <typename T, int V>
+struct OwnPlain {
+    const T* x;
+    static constexpr int VEC = V, NIN = 1;
+    __device__ __forceinline__ void init(int64_t) {}
+    __device__ __forceinline__ void load(int64_t at, float (&in)[NIN][VEC]) const { VecIO<T, V>::load(x + at, in[0]); }
+    __device__ __forceinline__ void finish(int64_t, float (&)[NIN][VEC]) const {}
+};
+template <typename D>
+__device__ __forceinline__ void store4_as16(D* p, const float (&v)[4]) {
+    const unsigned lo = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[0])) |
+                        ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[1])) << 16);
+    const unsigned hi = (unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[2])) |
+                        ((unsigned)__builtin_bit_cast(unsigned short, from_f32<D>(v[3])) << 16);
+    *reinterpret_cast<uint2*>(p) = make_uint2(lo, hi);
+}
+// fp32 x, summed as it is, with its 16-bit copy written (colsum_cast_partial)
+template <typename D>
+struct OwnCast {
+    const float* x;
+    D* x16;
+    static constexpr int VEC = 4, NIN = 1;
+    __device__ __forceinline__ void init(int64_t) {}
+    __device__ __forceinline__ void load(int64_t at, float (&in)[NIN][VEC]) const { VecIO<float, 4>::load(x + at, in[0]); }
+    __device__ __forceinline__ void finish(int64_t at, float (&in)[NIN][VEC]) const { store4_as16<D>(x16 + at, in[0]); }
+};
+// dx = dy * gelu'(u) in fp32, written as fp32 and as a 16-bit copy, summed (gelu_bwd_colsum_cast_partial)
+template <typename D>
+struct OwnGeluBwdCast {
+    const float* dy;
+    const float* u;
+    float* dx;
+    D* dx16;
+    static constexpr int VEC = 4, NIN = 2;
+    __device__ __forceinline__ void init(int64_t) {}
+    __device__ __forceinline__ void load(int64_t at, float (&in)[NIN][VEC]) const {
+        VecIO<float, 4>::load(dy + at, in[0]);
+        VecIO<float, 4>::load(u + at, in[1]);
+    }
+    __device__ __forceinline__ void finish(int64_t at, float (&in)[NIN][VEC]) const {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            in[0][j] = in[0][j] * gelu_grad_one(in[1][j]);
+            asm volatile("" : "+v"(in[0][j]));   // one fp32 value for the store, the copy and the sum
+        }
+        VecIO<float, 4>::store(dx + at, in[0]);
+        store4_as16<D>(dx16 + at, in[0]);
+    }
+};
+// dx = dy * gelu'(x + bias) in the storage type; what was stored is what is summed (bias_gelu_bwd_kernel)
+template <typename T, int V>
+struct OwnBiasGeluBwd {
+    const T* dy;
+    const T* x;
+    const float* bias;
+    T* dx;
+    float b[V];
+    static constexpr int VEC = V, NIN = 2;
+    __device__ __forceinline__ void init(int64_t col) {
+#pragma unroll
+        for (int j = 0; j < V; j++) b[j] = bias ? bias[col + j] : 0.f;
+    }
+    __device__ __forceinline__ void load(int64_t at, float (&in)[NIN][VEC]) const {
+        VecIO<T, V>::load(dy + at, in[0]);
+        VecIO<T, V>::load(x + at, in[1]);
+    }
+    __device__ __forceinline__ void finish(int64_t at, float (&in)[NIN][VEC]) const {
+#pragma unroll
+        for (int j = 0; j < V; j++) in[0][j] *= gelu_grad_one(in[1][j] + b[j]);
+        VecIO<T, V>::store_rounded(dx + at, in[0]);
+    }
+};
+
+constexpr int kOwnThreads = 1024, kOwnLanesPerRow = 8, kOwnRowsPerPass = kOwnThreads / kOwnLanesPerRow;
+
+template <int UNROLL, typename Src>
+__global__ __launch_bounds__(kOwnThreads) void colsum_owner_kernel(Src src_arg, float* __restrict__ out, int64_t rows,
+                                                                   int64_t cols, float scale) {
+    constexpr int VEC = Src::VEC, NIN = Src::NIN, RPP = kOwnRowsPerPass, CW = kOwnLanesPerRow * VEC;
+    __shared__ float slots[RPP][CW + 1];
+    Src src = src_arg;
+    const int lr = threadIdx.x % kOwnLanesPerRow, rr = threadIdx.x / kOwnLanesPerRow;
+    const int64_t col = (int64_t)blockIdx.x * CW + lr * VEC;
+    float acc[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++) acc[j] = 0.f;
+    if (col < cols) {
+        src.init(col);
+        int64_t r = rr;
+        for (; r + (UNROLL - 1) * RPP < rows; r += UNROLL * RPP) {
+            float in[UNROLL][NIN][VEC];
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) src.load((r + u * RPP) * cols + col, in[u]);
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) {
+                src.finish((r + u * RPP) * cols + col, in[u]);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc[j] += in[u][0][j];
+            }
+        }
+        for (; r < rows; r += RPP) {
+            float in[NIN][VEC];
+            src.load(r * cols + col, in);
+            src.finish(r * cols + col, in);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc[j] += in[0][j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) slots[rr][lr * VEC + j] = acc[j];
+    __syncthreads();
+    // 1024 / CW threads per column take every (1024 / CW)-th slot, then one thread per column takes those
+    constexpr int SLICES = kOwnThreads / CW;
+    static_assert(SLICES <= RPP, "the second stage reuses the slots");
+    const int c = threadIdx.x % CW, s = threadIdx.x / CW;
+    float t = 0.f;
+    for (int k = s; k < RPP; k += SLICES) t += slots[k][c];
+    __syncthreads();
+    slots[s][c] = t;
+    __syncthreads();
+    if (s == 0) {
+        float z = 0.f;
+        for (int k = 0; k < SLICES; k++) z += slots[k][c];
+        const int64_t oc = (int64_t)blockIdx.x * CW + c;
+        if (oc < cols) out[oc] = z * scale;
+    }
+}
+
+// Where one launch beats two (measured, see above): enough column blocks to occupy the chip, and for 4-byte elements
+// (32 columns per workgroup, half as many workgroups) and the bias-GELU backward only up to 1024 rows.  Depends on the shape and the element
+// size alone, so entries that promise each other's bits (br_hip_colsum / br_hip_colsum_cast /
+// br_hip_gelu_bwd_colsum_cast on fp32) always agree on the path.
+#ifndef BR_COLSUM_OWNER
+#define BR_COLSUM_OWNER 3   // bit 0: plain sums and sums with a copy; bit 1: the bias-GELU backward
+#endif
+bool colsum_owner_applies(int64_t rows, int64_t cols, int elem_bytes, int kind = 1) {
+    if (!(BR_COLSUM_OWNER & kind)) return false;
+    const int64_t cw = kOwnLanesPerRow * (elem_bytes == 4 ? 4 : 8);
+    const int64_t blocks = (cols + cw - 1) / cw;
+    if (cols % (elem_bytes == 4 ? 4 : 8) != 0 || blocks < 96 || blocks > 0x7fffffffLL) return false;
+    return (elem_bytes == 2 && kind == 1) || rows <= 1024;
+}
+
+template <int UNROLL, typename Src>
+int colsum_owner_launch(const Src& src, float* out, int64_t rows, int64_t cols, float scale, hipStream_t st) {
+    const int64_t cw = kOwnLanesPerRow * Src::VEC;
+    colsum_owner_kernel<UNROLL, Src><<<(unsigned)((cols + cw - 1) / cw), kOwnThreads, 0, st>>>(src, out, rows, cols, scale);
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
 // ------------------------------------------------------- transpose 0213
 // One 16-byte granule per thread, indexed by OUTPUT position so stores are
 // fully coalesced; loads are contiguous runs of s3 elements.
@@ -1042,6 +1204,18 @@ int br_hip_bias_gelu_bwd(const void* dy, const void* x, const float* bias, void*
         partial = (float*)workspace;
     }
     const bool al = aligned16(dy) && aligned16(x) && aligned16(dx);
+    if (dbias && al && colsum_owner_applies(rows, cols, dtype == BR_F32 ? 4 : 2, 2)) {
+        // gradient and bias gradient from one launch
+        if (dtype == BR_F32)
+            return colsum_owner_launch<2>(OwnBiasGeluBwd<float, 4>{(const float*)dy, (const float*)x, bias, (float*)dx},
+                                          dbias, rows, cols, dbias_scale, st);
+        if (dtype == BR_F16)
+            return colsum_owner_launch<2>(OwnBiasGeluBwd<__half, 8>{(const __half*)dy, (const __half*)x, bias, (__half*)dx},
+                                          dbias, rows, cols, dbias_scale, st);
+        return colsum_owner_launch<2>(OwnBiasGeluBwd<__hip_bfloat16, 8>{(const __hip_bfloat16*)dy, (const __hip_bfloat16*)x,
+                                                                        bias, (__hip_bfloat16*)dx},
+                                      dbias, rows, cols, dbias_scale, st);
+    }
     if (dtype == BR_F32 && al && cols % 4 == 0) {
         dim3 grid((unsigned)((cols / 4 + kBlock - 1) / kBlock), (unsigned)groups);
         bias_gelu_bwd_kernel<float, 4><<<grid, kBlock, 0, st>>>((const float*)dy, (const float*)x, bias,
@@ -1095,6 +1269,11 @@ int br_hip_colsum(const void* x, int dtype, float* out, int64_t rows, int64_t co
     float* partial = (float*)workspace;
     const int vec = dtype == BR_F32 ? 4 : 8;
     if (cols % vec == 0 && aligned16(x) && (cols * (dtype == BR_F32 ? 4 : 2)) % 16 == 0) {
+        if (colsum_owner_applies(rows, cols, dtype == BR_F32 ? 4 : 2)) {
+            if (dtype == BR_F32) return colsum_owner_launch<4>(OwnPlain<float, 4>{(const float*)x}, out, rows, cols, out_scale, st);
+            if (dtype == BR_F16) return colsum_owner_launch<4>(OwnPlain<__half, 8>{(const __half*)x}, out, rows, cols, out_scale, st);
+            return colsum_owner_launch<4>(OwnPlain<__hip_bfloat16, 8>{(const __hip_bfloat16*)x}, out, rows, cols, out_scale, st);
+        }
         const int64_t blocks_x = (cols / vec + kBlock - 1) / kBlock;
         const int rpb = colsum_vec_rows_per_block(rows, blocks_x);
         const int groups = (int)((rows + rpb - 1) / rpb);
@@ -1131,6 +1310,10 @@ int br_hip_colsum_cast(const float* x, float* out, void* x16, int x16_dtype, int
     if (cols % 4 != 0 || !aligned16(x) || (reinterpret_cast<uintptr_t>(x16) & 7u) != 0) return BR_ERR_TODO;
     if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
     hipStream_t st = as_stream(stream);
+    if (colsum_owner_applies(rows, cols, 4)) {
+        if (x16_dtype == BR_F16) return colsum_owner_launch<4>(OwnCast<__half>{x, (__half*)x16}, out, rows, cols, out_scale, st);
+        return colsum_owner_launch<4>(OwnCast<__hip_bfloat16>{x, (__hip_bfloat16*)x16}, out, rows, cols, out_scale, st);
+    }
     float* partial = (float*)workspace;
     const int64_t blocks_x = (cols / 4 + kBlock - 1) / kBlock;
     const int rpb = colsum_vec_rows_per_block(rows, blocks_x);
@@ -1156,6 +1339,12 @@ int br_hip_gelu_bwd_colsum_cast(const float* dy, const float* x, float* dx, floa
         return BR_ERR_TODO;
     if (!workspace || workspace_bytes < br_hip_colsum_workspace(rows, cols)) return BR_ERR_ATTR;
     hipStream_t st = as_stream(stream);
+    if (colsum_owner_applies(rows, cols, 4)) {
+        if (dx16_dtype == BR_F16)
+            return colsum_owner_launch<2>(OwnGeluBwdCast<__half>{dy, x, dx, (__half*)dx16}, out, rows, cols, out_scale, st);
+        return colsum_owner_launch<2>(OwnGeluBwdCast<__hip_bfloat16>{dy, x, dx, (__hip_bfloat16*)dx16}, out, rows, cols,
+                                      out_scale, st);
+    }
     float* partial = (float*)workspace;
     // same strips as br_hip_colsum_cast, hence the same summation order
     const int64_t blocks_x = (cols / 4 + kBlock - 1) / kBlock;

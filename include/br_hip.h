@@ -391,7 +391,9 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
  * of the projection's backward would round them) with the element strides of
  * q, k, v.  delta: fp32 scratch of
  * batch * heads * tokens entries (receives rowsum(d_o * o)).  Deterministic: one
- * pass accumulates dk / dv per key block, a second one dq per query block.
+ * pass accumulates dq per query block (and forms delta on the way), a second one
+ * dk / dv per key block.  dq, dk and dv must not be q, k, v, o or d_o themselves
+ * (BR_ERR_OUTPUT): the second pass still reads all five.
  * Same shape limits as the forward (BR_ERR_TODO otherwise). */
 int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o,
                           int dtype, const float* alibi, const int32_t* valid, const float* lse,

@@ -155,3 +155,11 @@ def test_flash_backward_against_the_unfused_chain(b, nh, t, valid, dtype, tdtype
     for bi in range(b):
         if 0 < valid[bi] < t:
             assert not host(gk)[bi, valid[bi]:].any() and not host(gv)[bi, valid[bi]:].any()
+    # delta is left behind as documented: rowsum(dO * O) per (batch, head, token)
+    want = (dg.float() * o.float()).sum(-1).permute(0, 2, 1)
+    assert bool(((delta - want).abs() <= 1e-5 * (want.abs() + want.pow(2).mean().sqrt()) + 1e-30).all())
+    # a gradient written over an operand the second pass still reads is refused, nothing runs
+    assert hip.load().br_hip_flash_attn_bwd(ptr(dq_), ptr(dk_), ptr(dv_), ptr(o), ptr(dg), dtype, ptr(alibi), ptr(dvalid),
+                                            ptr(lse), ptr(delta), ptr(dq_), ptr(gk), ptr(gv), dtype, *strides,
+                                            stream()) == -3
+    torch.cuda.synchronize()

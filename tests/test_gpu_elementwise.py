@@ -59,7 +59,8 @@ def test_bias_gelu_f16_headline_shape():
     assert_close(host(dbias), got_g.astype(np.float64).sum(0), RTOL, "dbias")
 
 
-@pytest.mark.parametrize("rows,cols,dtype", [(33, 1024, "f32"), (7, 100, "f32"), (5, 24, "f16"), (9, 31, "f16")])
+@pytest.mark.parametrize("rows,cols,dtype", [(33, 1024, "f32"), (7, 100, "f32"), (5, 24, "f16"), (9, 31, "f16"),
+                                             (130, 6152, "f16"), (300, 3080, "f32"), (512, 16384, "f16")])
 def test_bias_gelu_small_and_unaligned(rows, cols, dtype):
     rng = np.random.default_rng(2)
     np_t, code, t_t = (np.float32, F32, torch.float32) if dtype == "f32" else (np.float16, F16, torch.float16)
@@ -127,7 +128,7 @@ def test_transpose_0213_bit_exact(shape, eb):
     assert np.array_equal(host(y), np.ascontiguousarray(x.transpose(0, 2, 1, 3)))
 
 
-@pytest.mark.parametrize("rows,cols", [(2048, 4096), (77, 130), (1, 8)])
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (77, 130), (1, 8), (512, 4096), (1000, 3080)])
 def test_colsum(rows, cols):
     rng = np.random.default_rng(6)
     x = rng.standard_normal((rows, cols)).astype(np.float32)
@@ -137,7 +138,24 @@ def test_colsum(rows, cols):
     assert_close(host(out), x.astype(np.float64).sum(0), RTOL, "colsum")
 
 
-@pytest.mark.parametrize("rows,cols", [(2048, 4096), (300, 1000), (5, 8), (1, 4)])
+@pytest.mark.parametrize("rows,cols,dtype", [(2048, 12288, "f16"), (130, 6152, "f16"), (513, 16384, "bf16"),
+                                             (77, 6144, "bf16"), (1, 6144, "f16"), (40, 1024, "f16")])
+def test_colsum_16_bit(rows, cols, dtype):
+    """Column sums of 16-bit tensors (the bias gradient of a linear layer whose
+    output gradient is kept in 16 bits): shapes wide enough for the
+    single-launch form (a workgroup per 64 columns walking all rows; ragged
+    last block, rows that do not fill a pass) and one that takes two launches."""
+    from gpu_util import BF16
+    rng = np.random.default_rng(61)
+    t, code = (torch.float16, F16) if dtype == "f16" else (torch.bfloat16, BF16)
+    x = torch.from_numpy(rng.standard_normal((rows, cols)).astype(np.float32)).cuda().to(t)
+    out = empty(cols)
+    ws = workspace(hip.load().br_hip_colsum_workspace(rows, cols))
+    call("br_hip_colsum", ptr(x), code, ptr(out), rows, cols, 0.5, ptr(ws), ws.numel(), stream())
+    assert_close(host(out), 0.5 * x.float().cpu().numpy().astype(np.float64).sum(0), RTOL, "colsum " + dtype)
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (300, 1000), (5, 8), (1, 4), (512, 4096), (300, 3080), (1, 3072)])
 def test_colsum_cast_equals_colsum_plus_cast(rows, cols):
     """One pass giving the column sums and the fp16 copy: the sums must equal
     br_hip_colsum's bit for bit (same strips, same order), the copy the cast's."""
@@ -321,7 +339,7 @@ def test_memset_fills_exactly_the_requested_bytes(offset, nbytes):
 
 
 @pytest.mark.parametrize("dtype,tdtype", [(F16, torch.float16), (BF16, torch.bfloat16)])
-@pytest.mark.parametrize("rows,cols", [(2048, 16384), (37, 64), (5, 1000)])
+@pytest.mark.parametrize("rows,cols", [(2048, 16384), (37, 64), (5, 1000), (512, 16384), (300, 3080)])
 def test_gelu_bwd_colsum_cast_equals_the_separate_kernels(rows, cols, dtype, tdtype):
     """One pass producing the GELU gradient, its 16-bit copy and its column
     sums: each bit for bit what br_hip_gelu_bwd followed by br_hip_colsum_cast
