@@ -532,6 +532,208 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     }
 }
 
+// ---- the same product with workgroups that stay -------------------------------------------------
+// 32 workgroups per XCD walk the tiles of that XCD's share instead of one workgroup being launched per tile; the
+// tile order, the K walk and the order of every sum are those of gemm_dtl_kernel, so the bits are too.  What it
+// buys: a workgroup issues the first two K stages of its NEXT tile before the C stores of the current one, and lets
+// up to 63 of those stores stay in flight through the next tile's first K step -- the 2.3 us a fresh workgroup
+// spends being launched and waiting for its first operand tile disappear behind the epilogue.  Measured on products
+// of the BLOOM-7B1 block (same run, before / after): weight gradient [16384 x 4096] from K = 2048 253 -> 245 us,
+// from K = 512 99 -> 95 us, [4096 x 4096] 66.2 -> 64.6, h -> 4h forward 241 -> 237.
+// Memory operations complete in issue order on this target, which is what the partial waits rest on: after the 16
+// operand loads of the next tile come the wave's 128 stores, so "at most 63 outstanding" means the loads are in.
+// Plain products only: 256 x 256 tiles, all of them interior (m, n multiples of 256), one batch, no bias, nothing
+// accumulated, no second output (walk_applies); everything else takes gemm_dtl_kernel.
+template <int CT, bool A_KSTR, bool B_KSTR, typename TC>
+__global__ __launch_bounds__(512) void gemm_dtl_walk_kernel(GemmArgs g) {
+    constexpr int BM = 256, BN = 256, WM = 64, WN = 128, KT = 64, STAGES = 2;
+    constexpr int WAVES = (BM / WM) * (BN / WN);
+    constexpr int FM = WM / 32, FN = WN / 32, KS = KT / 16;
+    using TA = DtlTile<BM, KT, WAVES, A_KSTR>;
+    using TB = DtlTile<BN, KT, WAVES, B_KSTR>;
+    constexpr int kStageBytes = TA::kBytes + TB::kBytes;
+    constexpr int kLoads = TA::kPerWave + TB::kPerWave;
+    static_assert(FM * FN * 16 >= 63, "the partial wait counts on at least 63 stores per wave and tile");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[STAGES * kStageBytes];
+    const lds_byte* lds = (const lds_byte*)lds_raw;
+    const unsigned lds0 = (unsigned)(unsigned long long)lds;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / (BN / WN), wn = wave % (BN / WN);
+    // workgroup ids are dealt to the 8 XCDs round-robin: this one is number `slot` of `slots` on XCD `xcd`, whose
+    // share of the tile order is [xcd * per_xcd, (xcd + 1) * per_xcd), as in tile_coords
+    const int per_xcd = g.tiles_m * g.tiles_n / 8;
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, slots = gridDim.x >> 3;
+    const int my_tiles = (per_xcd - slot + slots - 1) / slots;
+    const int nk = (int)(g.k / KT);
+
+    unsigned fa_off[FM][KS], fb_off[FN][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+        for (int i = 0; i < FM; i++) fa_off[i][ks] = TA::frag_offset(wm * WM + i * 32, ks, lane);
+#pragma unroll
+        for (int j = 0; j < FN; j++) fb_off[j][ks] = TA::kBytes + TB::frag_offset(wn * WN + j * 32, ks, lane);
+    }
+    // interior tiles: a lane's chunk offsets inside the operand tiles are the same for every tile
+    unsigned a_off[TA::kPerWave], b_off[TB::kPerWave];
+#pragma unroll
+    for (int q = 0; q < TA::kPerWave; q++) a_off[q] = TA::source_offset(q, wave, lane, g.lda, 0, g.m);
+#pragma unroll
+    for (int q = 0; q < TB::kPerWave; q++) b_off[q] = TB::source_offset(q, wave, lane, g.ldb, 0, g.n);
+    const long long a_step = A_KSTR ? 2 * KT * g.lda : 2 * KT;
+    const long long b_step = B_KSTR ? 2 * KT * g.ldb : 2 * KT;
+
+    const unsigned char* a_src = nullptr;
+    const unsigned char* b_src = nullptr;
+    int until_wrap = 0;
+    long long row0 = 0, col0 = 0;
+    auto setup = [&](int it) {   // the it-th tile of this workgroup: origins and the start of its K walk
+        int tm, tn;
+        tile_in_order(g, xcd * per_xcd + it * slots + slot, tm, tn);
+        tm = __builtin_amdgcn_readfirstlane(tm);
+        tn = __builtin_amdgcn_readfirstlane(tn);
+        row0 = (long long)tm * BM;
+        col0 = (long long)tn * BN;
+        const int first = (int)(k_walk_start(row0, col0, g.k) / KT);
+        a_src = reinterpret_cast<const unsigned char*>(g.a) + 2 * (A_KSTR ? row0 : row0 * g.lda) + first * a_step;
+        b_src = reinterpret_cast<const unsigned char*>(g.b) + 2 * (B_KSTR ? col0 : col0 * g.ldb) + first * b_step;
+        until_wrap = nk - first;
+    };
+    auto issue = [&](int tile) {
+        const unsigned dst = lds0 + (unsigned)(tile % STAGES) * kStageBytes + (unsigned)wave * 1024u;
+#pragma unroll
+        for (int q = 0; q < kLoads; q++) {
+            if (q < TA::kPerWave) dtl_load(dst + q * WAVES * 1024, a_off[q], a_src);
+            else dtl_load(dst + TA::kBytes + (q - TA::kPerWave) * WAVES * 1024, b_off[q - TA::kPerWave], b_src);
+        }
+        const bool wraps = --until_wrap == 0;
+        a_src += wraps ? a_step - nk * a_step : a_step;
+        b_src += wraps ? b_step - nk * b_step : b_step;
+    };
+    f32x16 acc[FM][FN];
+    auto step = [&](const u32x4 (&fa)[FM], const u32x4 (&fb)[FN], u32x4 (&na)[FM], u32x4 (&nb)[FN], int tile, int ks) {
+        const lds_byte* stage = lds + (tile % STAGES) * kStageBytes;
+#pragma unroll
+        for (int idx = 0; idx < FM * FN; idx++) {
+            const int i = idx % FM, j = idx / FM;
+            if (idx == 0) nb[0] = TB::fragment(stage, fb_off[0][ks]);
+            else if (idx <= FM) na[idx - 1] = TA::fragment(stage, fa_off[idx - 1][ks]);
+            else if (idx < FM + FN) nb[idx - FM] = TB::fragment(stage, fb_off[idx - FM][ks]);
+            acc[i][j] = Cvt<CT>::mfma(fa[i], fb[j], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    setup(0);
+    issue(0);
+    if (nk > 1) issue(1);
+    for (int it = 0; it < my_tiles; it++) {
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+        // K stage 0 of this tile has to be in LDS.  First tile: nothing but its two stages is outstanding.  Later
+        // tiles: both stages were issued ahead of the previous tile's stores, so they have landed once at most 63
+        // operations (all of them stores) are outstanding.
+        if (nk == 1) wait_vmem<0>();
+        else if (it == 0) wait_vmem<kLoads>();
+        else wait_vmem<63>();
+        __syncthreads();
+        u32x4 fa0[FM], fb0[FN], fa1[FM], fb1[FN];
+#pragma unroll
+        for (int i = 0; i < FM; i++) fa0[i] = TA::fragment(lds, fa_off[i][0]);
+#pragma unroll
+        for (int j = 0; j < FN; j++) fb0[j] = TB::fragment(lds, fb_off[j][0]);
+        __builtin_amdgcn_sched_barrier(0);
+        for (int t = 0; t < nk; t++) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                u32x4(&fa_now)[FM] = (ks & 1) ? fa1 : fa0;
+                u32x4(&fb_now)[FN] = (ks & 1) ? fb1 : fb0;
+                u32x4(&fa_next)[FM] = (ks & 1) ? fa0 : fa1;
+                u32x4(&fb_next)[FN] = (ks & 1) ? fb0 : fb1;
+                if (ks + 1 < KS) {
+                    step(fa_now, fb_now, fa_next, fb_next, t, ks + 1);
+                } else {
+                    // K stage t+1 has to be in LDS: the only loads in flight, except during step 0 of a later tile,
+                    // when stage 1 is already in and up to 63 of the previous tile's stores may go on draining
+                    if (t == 0 && it > 0) wait_vmem<63>(); else wait_vmem<0>();
+                    __syncthreads();
+                    if (t + STAGES < nk) issue(t + STAGES);
+                    __builtin_amdgcn_sched_barrier(0);
+                    step(fa_now, fb_now, fa_next, fb_next, t + 1, 0);
+                }
+            }
+        }
+        // Every wave is past the last barrier of the K loop and nothing in LDS is read for its value any more (the
+        // loop's trailing fragment reads fetch a stage that does not exist): the next tile's first stages may go.
+        const long long st_row0 = row0, st_col0 = col0;
+        if (it + 1 < my_tiles) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            setup(it + 1);
+            issue(0);
+            if (nk > 1) issue(1);
+        }
+        // acc[i][j][v] is C[row, col] with row = wm*WM + i*32 + (v/4)*8 + (lane/32)*4 + v%4, col = wn*WN + j*32 + lane%32
+        const unsigned lane_bytes = (unsigned)(((lane >> 5) * 4 * g.ldc + (lane & 31)) * (long long)sizeof(TC));
+        const long long tile_at = (st_row0 + wm * WM) * g.ldc + st_col0 + wn * WN;
+        char* const c_tile = reinterpret_cast<char*>(static_cast<TC*>(g.c) + tile_at);
+        float alpha = g.alpha;
+        asm volatile("" : "+v"(alpha));
+#pragma unroll
+        for (int blk = 0; blk < FM * FN; blk++) {
+            const int i = blk / FN, j = blk % FN;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float o = alpha * acc[i][j][v] + 0.f;   // the plain epilogue's expression with its bias of zero
+                if (sizeof(TC) == 2) asm volatile("" : "+v"(o));   // one fp32 value, then one rounding (see gemm_dtl_kernel)
+                c_store<TC>(reinterpret_cast<TC*>(c_tile + (i * 32 + (v >> 2) * 8 + (v & 3)) * g.ldc * (long long)sizeof(TC) +
+                                                  j * 32 * sizeof(TC) + lane_bytes), o);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
+// Whether the walking form takes a product the plan has put on 256 x 256 tiles.
+#ifndef BR_DTL_WALK
+#define BR_DTL_WALK 1   // 0: every product on one workgroup per tile (for an A/B build)
+#endif
+inline bool walk_applies(const GemmArgs& g, long long batch) {
+    if (!BR_DTL_WALK) return false;
+    const long long tiles = (g.m / 256) * (g.n / 256);
+    return batch == 1 && g.m % 256 == 0 && g.n % 256 == 0 && g.k % 64 == 0 && tiles >= 256 && tiles % 8 == 0 &&
+           tiles <= 0x7fffffffLL && !g.bias && !g.accumulate && !g.c2 && !g.addend && g.splits == 1;
+}
+
+template <int CT>
+int launch_dtl_walk(GemmArgs g, const Problem& p, hipStream_t st) {
+    g.tiles_m = (int)(g.m / 256);
+    g.tiles_n = (int)(g.n / 256);
+    using F16 = __half;
+    using BF16 = __hip_bfloat16;
+#define BR_DTL_WALK_CASE(AK, BK_)                                                        \
+    if (p.a_kstr == AK && p.b_kstr == BK_) {                                             \
+        if (p.c_dtype == BR_F32)                                                         \
+            gemm_dtl_walk_kernel<CT, AK, BK_, float><<<256, 512, 0, st>>>(g);            \
+        else if (CT == BR_GEMM_F16)                                                      \
+            gemm_dtl_walk_kernel<CT, AK, BK_, F16><<<256, 512, 0, st>>>(g);              \
+        else                                                                             \
+            gemm_dtl_walk_kernel<CT, AK, BK_, BF16><<<256, 512, 0, st>>>(g);             \
+    }
+    BR_DTL_WALK_CASE(false, false)
+    BR_DTL_WALK_CASE(false, true)
+    BR_DTL_WALK_CASE(true, false)
+    BR_DTL_WALK_CASE(true, true)
+#undef BR_DTL_WALK_CASE
+    BR_HIP_LAUNCH_CHECK();
+    return BR_OK;
+}
+
 // ---- host-side dispatch -------------------------------------------------------
 template <int CT, int BM, int BN, int WM, int WN, int KT, int ST>
 int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
@@ -726,6 +928,7 @@ int launch_dtl(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
         return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(tail, p, batch, st);
     }
     const int pick = plan.config;
+    if (pick == 0 && walk_applies(g, batch)) return launch_dtl_walk<CT>(g, p, st);
     if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
     if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
     if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);

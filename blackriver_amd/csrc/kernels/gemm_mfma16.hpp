@@ -275,20 +275,12 @@ template <>
 __device__ __forceinline__ void c_store<__hip_bfloat16>(__hip_bfloat16* p, float v) { *p = __float2bfloat16(v); }
 
 
-// Workgroup id -> (batch, tile_m, tile_n).
-__device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch, int& tm, int& tn) {
-    const long long nb = gridDim.x;
-    long long id = blockIdx.x;
-    // ids are dealt to the 8 XCDs round-robin; make each XCD's share contiguous
-    const long long per_xcd = nb / 8;
-    if (per_xcd > 0 && id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
-    const long long per_batch = (long long)g.tiles_m * g.tiles_n;
-    batch = id / per_batch;
-    const int rem = (int)(id % per_batch);
-    // Panels of GN tile columns; inside a panel, blocks of GM x gn tiles with m
-    // fastest: the ~32 workgroups an XCD runs at a time cover a GM x GN block and
-    // share GM + GN operand strips in its L2 (8 x 4: 12 strips for 32 tiles; a
-    // column-first walk down a tall product would touch 33).
+// Tile number `rem` (0 .. tiles_m * tiles_n - 1) of one batch in the order workgroups take them.
+// Panels of GN tile columns; inside a panel, blocks of GM x gn tiles with m
+// fastest: the ~32 workgroups an XCD runs at a time cover a GM x GN block and
+// share GM + GN operand strips in its L2 (8 x 4: 12 strips for 32 tiles; a
+// column-first walk down a tall product would touch 33).
+__device__ __forceinline__ void tile_in_order(const GemmArgs& g, int rem, int& tm, int& tn) {
     const int GM = g.tiles_m < 8 ? g.tiles_m : 8;
     const int GN = 32 / GM > 4 ? 32 / GM : 4;
     const int group = rem / (GN * g.tiles_m);
@@ -300,6 +292,19 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch,
     const int gm = g.tiles_m - blk * GM < GM ? g.tiles_m - blk * GM : GM;
     tm = blk * GM + within % gm;
     tn = first_n + within / gm;
+}
+
+// Workgroup id -> (batch, tile_m, tile_n).
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, long long& batch, int& tm, int& tn) {
+    const long long nb = gridDim.x;
+    long long id = blockIdx.x;
+    // ids are dealt to the 8 XCDs round-robin; make each XCD's share contiguous
+    const long long per_xcd = nb / 8;
+    if (per_xcd > 0 && id < per_xcd * 8) id = (id % 8) * per_xcd + id / 8;
+    const long long per_batch = (long long)g.tiles_m * g.tiles_n;
+    batch = id / per_batch;
+    const int rem = (int)(id % per_batch);
+    tile_in_order(g, rem, tm, tn);
 }
 
 // Where a tile starts its walk over K (an element index, a multiple of 64; the walk wraps round at the end of K).

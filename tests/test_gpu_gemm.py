@@ -194,6 +194,28 @@ def test_gemm_direct_to_lds_at_linear_layer_shape():
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("m,n,k,c_dt", [
+    (2048, 8192, 192, F32),     # 256 tiles: one per workgroup, three K steps
+    (2048, 16384, 128, F16),    # 512 tiles: two per workgroup, 16-bit C
+    (3072, 16384, 64, F32),     # 768 tiles of a single K step
+    (2816, 6144, 320, F32),     # 264 tiles: 33 per XCD for 32 workgroups, one of them walks twice
+])
+def test_gemm_workgroups_that_walk_the_tiles(ta, tb, m, n, k, c_dt):
+    """Plain products (no bias, nothing accumulated) of 256 or more interior
+    256 x 256 tiles run on 256 workgroups that each walk several tiles, loading
+    the next tile's first K stages ahead of the current tile's stores.  Against
+    fp64, and for an fp32 C bit for bit against the same product with a bias of
+    zeros, which takes the one-workgroup-per-tile kernel."""
+    rng = np.random.default_rng(31)
+    print("case ta=%d tb=%d m=%d n=%d k=%d c_dt=%d" % (ta, tb, m, n, k, c_dt), flush=True)
+    a, b = operands(rng, ta, tb, m, n, k)
+    got, ref = run_gemm(ta, tb, m, n, k, a, b, F16, F16, c_dt, hip.GEMM_F16, alpha=0.5)
+    assert_close(got, ref, 2e-2, "walking workgroups")
+    per_tile, _ = run_gemm(ta, tb, m, n, k, a, b, F16, F16, c_dt, hip.GEMM_F16, alpha=0.5, bias=np.zeros(n, np.float32))
+    assert np.array_equal(got, per_tile)
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
 @pytest.mark.parametrize("n,c_dt", [(12288, F16), (12248, F32)])
 def test_gemm_round_and_a_half_of_tiles(ta, tb, n, c_dt):
     """[2048 x 12288] from K = 1024: 384 tiles of 256 x 256 are a round and a
