@@ -236,7 +236,7 @@ def roofline_leg(hip, timer, torch, full):
     f32, f16 = hip.F32, hip.F16
     sec, flop = gemm_case(hip, timer, torch, 1, 0, F, H, N, f16, f16, f32, iters=60, sets=4, warmup=150)
     traffic, source = roofline_traffic()
-    roof = {"bound": "mfma", "kernel": "gemm_dtl_kernel 256x256x64 (A fp16 [k,m], B fp16 [k,n], C fp32)",
+    roof = {"bound": "mfma", "kernel": "gemm_dtl_walk_kernel, 256x256x64 tiles (A fp16 [k,m], B fp16 [k,n], C fp32)",
             "shape": "m=%d n=%d k=%d" % (F, H, N), "achieved": flop / sec / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
             "unit": "TFLOP/s", "frac": flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, "us_per_launch": sec * 1e6,
             "traffic": traffic, "traffic_source": source}
