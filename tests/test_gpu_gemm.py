@@ -215,6 +215,31 @@ def test_gemm_workgroups_that_walk_the_tiles(ta, tb, m, n, k, c_dt):
     assert np.array_equal(got, per_tile)
 
 
+@pytest.mark.parametrize("k", [512, 2048])
+def test_gemm_walking_workgroups_at_the_weight_gradient_shape(k):
+    """dW[16384, 4096] = dy[k, 16384]^T . x[k, 4096] (1024 tiles, four per
+    workgroup) at both token counts of the benchmarks: bit for bit the
+    one-workgroup-per-tile kernel (taken with a bias of zeros), three launches
+    in a row on rotating operands, and a sample of rows against fp64."""
+    torch.manual_seed(k)
+    m, n = 16384, 4096
+    sets = [(torch.randn((k, m), device="cuda").half(), torch.randn((k, n), device="cuda").half()) for _ in range(3)]
+    zeros = torch.zeros(n, device="cuda")
+    for a, b in sets:
+        outs = []
+        for bias in (None, zeros):
+            c = torch.full((m, n), float("nan"), device="cuda")
+            call("br_hip_gemm", 1, 0, m, n, k, 0.25, ptr(a), F16, m, 0, ptr(b), F16, n, 0, 0, ptr(c), F32, n, 0, ptr(bias),
+                 1, hip.GEMM_F16, stream())
+            outs.append(c)
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1])
+        rows = torch.arange(0, m, 257, device="cuda")
+        ref = 0.25 * (a[:, rows].double().t() @ b.double())
+        err = (outs[0][rows].double() - ref).abs()
+        assert bool((err <= 1e-5 * (ref.abs() + ref.pow(2).mean().sqrt()) * (k ** 0.5)).all())
+
+
 @pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
 @pytest.mark.parametrize("n,c_dt", [(12288, F16), (12248, F32)])
 def test_gemm_round_and_a_half_of_tiles(ta, tb, n, c_dt):
