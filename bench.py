@@ -350,7 +350,27 @@ def elementwise_leg(hip, timer, torch):
     sec = timer.run(lambda i: hip.call("br_hip_bias_gelu_bwd", vp(dys[i % nb]), vp(xs[i % nb]), vp(bias), vp(ys[i % nb]),
                                        vp(dbias), hip.F16, rows, cols, 1.0, vp(ws), ws.numel(), st), 200, 10, blocker)
     rec("bias_gelu_bwd [2048,16384] f16 (+dbias)", sec, 3 * rows * cols * 2)
-    del xs, ys, dys, block_buf
+    del xs, ys, dys
+
+    # ALiBi + causal / padding mask + softmax over the scores of config C4 in one pass (the kernel the word machine
+    # puts in place of `op.add op.add op.softmax`), and the softmax backward of the same shape
+    heads = NH
+    ss = [torch.randn((B, heads, T, T), device="cuda") for _ in range(4)]
+    pp = [torch.empty_like(x) for x in ss]
+    alibi = torch.empty((heads, T), device="cuda")
+    xmask = torch.empty((B, T, T), device="cuda")
+    mask = torch.ones((B, T), device="cuda", dtype=torch.int32)
+    mask[-1, T - T // 4:] = 0
+    hip.call("br_hip_alibi_table", vp(alibi), heads, T, st)
+    hip.call("br_hip_xmask_table", vp(mask), vp(xmask), B, T, st)
+    sec = timer.run(lambda i: hip.call("br_hip_alibi_masked_softmax_fwd", vp(ss[i % 4]), vp(alibi), vp(xmask), vp(pp[i % 4]),
+                                       B, heads, T, T, st), 100, 10, blocker)
+    rec("alibi_masked_softmax_fwd [4,32,512,512] f32", sec, 2 * B * heads * T * T * 4 + B * T * T * 4)
+    dd = [torch.empty_like(x) for x in ss]
+    sec = timer.run(lambda i: hip.call("br_hip_softmax_bwd", vp(ss[i % 4]), vp(pp[i % 4]), vp(dd[i % 4]),
+                                       B * heads * T, T, st), 100, 10, blocker)
+    rec("softmax_bwd [65536,512] f32", sec, 3 * B * heads * T * T * 4)
+    del ss, pp, dd, block_buf
 
     rows, vocab = 2048, V
     logits = torch.randn((rows, vocab), device="cuda") * 2.0
@@ -421,11 +441,12 @@ def cpu_baseline_leg():
 
 
 def cpu_kernel_rows(orc):
-    """The memory-bound kernels of configurations C1-C3 on the host cores (the
-    oracle's restatements, all threads): wall time and the same algorithmic
-    bytes per second the GPU rows quote.  C1 and C2 run at full size, C3 on a
-    64-row sample of its 2048 rows (1 MB per row; the kernels are row-parallel,
-    so the rate carries over).  A baseline to read the GPU rows against, never
+    """The memory-bound kernels of configurations C1-C3 and the masked softmax
+    of C4 on the host cores (the oracle's restatements, all threads): wall time
+    and the same algorithmic bytes per second the GPU rows quote.  C1 and C2 run
+    at full size, the softmax on one of the four sequences, C3 on a 64-row
+    sample of its 2048 rows (1 MB per row; the kernels are row-parallel, so the
+    rate carries over).  A baseline to read the GPU rows against, never
     a target."""
     rng = np.random.default_rng(0)
     rows = {}
@@ -459,6 +480,16 @@ def cpu_kernel_rows(orc):
     rec("bias_gelu_fwd [2048,16384]", timed(lambda: orc.bias_gelu_fwd(x, bias)), 2 * r * c * 2, "fp32 storage on the host")
     rec("bias_gelu_bwd [2048,16384] (+dbias)", timed(lambda: orc.bias_gelu_bwd(dy, x, bias)), 3 * r * c * 2,
         "fp32 storage on the host")
+    # the scores of one sequence of config C4 (a quarter of its batch): the reference's three operators in a row
+    # (two broadcast additions and the softmax), then the softmax backward
+    b1, nh, t = 1, NH, T
+    s = rng.standard_normal((b1, nh, t, t)).astype(np.float32)
+    al = orc.alibi(nh, t).reshape(1, nh, 1, t)
+    xm = orc.xmask(np.ones((b1, t), np.int32)).reshape(b1, 1, t, t)
+    p = orc.softmax_fwd(orc.add_bcast(orc.add_bcast(s, al), xm))
+    rec("alibi_masked_softmax_fwd [4,32,512,512] f32", timed(lambda: orc.softmax_fwd(orc.add_bcast(orc.add_bcast(s, al), xm))),
+        2 * b1 * nh * t * t * 4 + b1 * t * t * 4, "one of the 4 sequences; three host operators in a row")
+    rec("softmax_bwd [65536,512] f32", timed(lambda: orc.softmax_bwd(s, p)), 3 * b1 * nh * t * t * 4, "one of the 4 sequences")
     r, v = 64, V
     logits = (2.0 * rng.standard_normal((r, v))).astype(np.float32)
     target = rng.integers(0, v, r).astype(np.int32)

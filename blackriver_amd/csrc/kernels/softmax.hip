@@ -29,6 +29,25 @@ struct RowBias {
     int heads, tq;
 };
 
+// Scores, probabilities and their gradients are read once and written once: streaming (non-temporal) accesses,
+// measured at [4,32,512,512] fp32 on one box: forward 55.4 us plain, 54.5 with streaming loads, 51.0 with streaming
+// stores too; backward 71 / 66.6 / 62.4.
+#ifndef BR_SM_STREAM
+#define BR_SM_STREAM 7   // one-wave-per-row kernels: bit 0 streaming loads, bit 1 streaming stores (forward), bit 2 (backward)
+#endif
+__device__ __forceinline__ float4 sm_load(const float4* p) {
+#if BR_SM_STREAM & 1
+    return load_stream(p);
+#else
+    return *p;
+#endif
+}
+template <int BIT>
+__device__ __forceinline__ void sm_store(float4* p, const float4& v) {
+    if (BR_SM_STREAM & BIT) store_stream(p, v);
+    else *p = v;
+}
+
 // exp(x - m) for x <= m, via the hardware exp2
 __device__ __forceinline__ float exp_sub(float x, float m) { return __expf(x - m); }
 
@@ -44,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void softmax_fwd_wave(const float* __restri
 #pragma unroll
     for (int i = 0; i < VPL; i++) {
         const int idx = lane + i * kWave;
-        v[i] = idx < cols4 ? xr[idx] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+        v[i] = idx < cols4 ? sm_load(xr + idx) : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     }
     if (MODE != kPlain) {
         // row = (b * heads + h) * tq + q
@@ -109,7 +128,7 @@ __global__ __launch_bounds__(kBlock) void softmax_fwd_wave(const float* __restri
         if (idx < cols4) {
             float4 o = make_float4(v[i].x * inv, v[i].y * inv, v[i].z * inv, v[i].w * inv);
             store4_as16(y16, row * cols4 + idx, o);
-            yr[idx] = o;
+            sm_store<2>(yr + idx, o);
         }
     }
 }
@@ -129,8 +148,8 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_wave(const float* __restri
     for (int i = 0; i < VPL; i++) {
         const int idx = lane + i * kWave;
         const bool ok = idx < cols4;
-        g[i] = ok ? gr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
-        p[i] = ok ? yr[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+        g[i] = ok ? sm_load(gr + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
+        p[i] = ok ? sm_load(yr + idx) : make_float4(0.f, 0.f, 0.f, 0.f);
         dot += (g[i].x * p[i].x + g[i].y * p[i].y) + (g[i].z * p[i].z + g[i].w * p[i].w);
     }
     dot = wave_sum(dot);
@@ -142,7 +161,7 @@ __global__ __launch_bounds__(kBlock) void softmax_bwd_wave(const float* __restri
             float4 o = make_float4(p[i].x * (g[i].x - dot), p[i].y * (g[i].y - dot), p[i].z * (g[i].z - dot),
                                    p[i].w * (g[i].w - dot));
             store4_as16(dx16, row * cols4 + idx, o);
-            if (dx) dr[idx] = o;  // dx == nullptr: only the 16-bit gradient is wanted
+            if (dx) sm_store<4>(dr + idx, o);  // dx == nullptr: only the 16-bit gradient is wanted
         }
     }
 }
