@@ -413,7 +413,7 @@ def copy_leg(hip, timer, torch):
     def fn(i):
         hip.call("br_hip_cast", ctypes.c_void_p(src.data_ptr()), hip.F32, ctypes.c_void_p(dst.data_ptr()), hip.F32, n, st)
     sec = timer.run(fn, 10, 2)
-    return {"kernel": "cast_x8_kernel<float, float>", "bytes_read": 4 * n, "bytes_written": 4 * n,
+    return {"kernel": "copy_x16_kernel", "bytes_read": 4 * n, "bytes_written": 4 * n,
             "us": sec * 1e6, "GB/s": 8 * n / sec / 1e9}
 
 

@@ -353,7 +353,7 @@ int stage_rows(const float* src, long long ld, long long stride, long long rows,
                void* dst, int compute, hipStream_t st) {
     const long long total = batch * rows * cols;
     if (ld == cols && (batch == 1 || stride == rows * cols) && total % 8 == 0 && aligned16(src) && aligned16(dst)) {
-        const unsigned grid = grid_for(total / 8, 256, 1 << 14);
+        const unsigned grid = grid_for(total / 8, 256);
         if (compute == BR_GEMM_F16)
             stage_flat_kernel<false><<<grid, 256, 0, st>>>(reinterpret_cast<const float4*>(src),
                                                            static_cast<gemm16::u32x4*>(dst), total / 8);
@@ -365,7 +365,7 @@ int stage_rows(const float* src, long long ld, long long stride, long long rows,
     }
     const bool vec = cols % 4 == 0 && ld % 4 == 0 && stride % 4 == 0 && aligned16(src) && aligned16(dst);
     const long long work = batch * rows * (vec ? cols / 4 : cols);
-    const unsigned grid = grid_for(work, 256, 1 << 16);
+    const unsigned grid = grid_for(work, 256);
     if (compute == BR_GEMM_F16) {
         if (vec) stage_rows_kernel<__half, true><<<grid, 256, 0, st>>>(src, ld, stride, rows, cols, batch, (__half*)dst);
         else stage_rows_kernel<__half, false><<<grid, 256, 0, st>>>(src, ld, stride, rows, cols, batch, (__half*)dst);
@@ -537,7 +537,7 @@ int staged_impl(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float
                                    compute, stream);
         if (rc != BR_OK) return rc;
         const long long mn4 = m * n / 4;
-        splitk_reduce_kernel<<<grid_for(mn4, 256, 1 << 14), 256, 0, st>>>(reinterpret_cast<const float4*>(part),
+        splitk_reduce_kernel<<<grid_for(mn4, 256), 256, 0, st>>>(reinterpret_cast<const float4*>(part),
                                                                         splits, mn4, n / 4, alpha, bias,
                                                                         accumulate ? (addend ? addend : c) : nullptr,
                                                                         c, c_dtype, ldc);
