@@ -42,6 +42,7 @@
 // operands rows % 8 == 0.  Rows past the end of an operand are redirected to a
 // valid row; their products land in rows / columns of C that are never stored.
 #pragma once
+#include <mutex>
 #include <type_traits>
 
 #include "gemm_mfma16.hpp"
@@ -161,11 +162,13 @@ struct DtlTile {
 // (every slice writing, one reading them all) this form measured slower than partials written with ordinary
 // stores and summed by a second kernel, which is what products with more slices use (gemm.hip).
 // The counters live in the library, start at zero and are put back to zero by the second arrival, so a launch needs
-// no clearing pass; two products split at the same time on different streams of one device would share them and
-// must not overlap.
+// no clearing pass.  There is one set per stream (kSplitSlots of them, handed out in the order streams first ask:
+// split_slot_of): products on one stream run one after the other and may share a set, products split at the same
+// time on different streams meet through different sets; a stream beyond the last set gets no split.
 constexpr int kMaxSplitTiles = 8192;
-static __device__ unsigned dtl_tickets[kMaxSplitTiles];
-static __device__ unsigned dtl_arrived[kMaxSplitTiles];
+constexpr int kSplitSlots = 8;
+static __device__ unsigned dtl_tickets[kSplitSlots][kMaxSplitTiles];
+static __device__ unsigned dtl_arrived[kSplitSlots][kMaxSplitTiles];
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 // The wait states after the store are part of the statement: a store of more than 64 bits reads its data
@@ -359,7 +362,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
         __syncthreads();
         unsigned* const drawn = reinterpret_cast<unsigned*>(lds_raw);
         if (threadIdx.x == 0)
-            *drawn = __hip_atomic_fetch_add(&dtl_tickets[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *drawn = __hip_atomic_fetch_add(&dtl_tickets[g.split_slot][tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         const bool last = *drawn == 1u;
         // Quad q of accumulator block (i, j) of thread t sits at quad index ((i*FN + j)*4 + q)*THREADS + t of the
@@ -382,7 +385,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
             wait_vmem<0>();   // this thread's stores have reached the level every XCD sees
             __syncthreads();  // ... and so have every other thread's of this workgroup
             if (threadIdx.x == 0)
-                __hip_atomic_fetch_add(&dtl_arrived[tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(&dtl_arrived[g.split_slot][tile_id], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             return;
         }
         // The second to draw: the other slice drew first, so it is past its K loop and on its way through the few
@@ -392,7 +395,7 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
         if (threadIdx.x == 0) {
             unsigned seen = 0;
             for (int spin = 0; spin < (1 << 22); spin++) {
-                seen = __hip_atomic_load(&dtl_arrived[tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                seen = __hip_atomic_load(&dtl_arrived[g.split_slot][tile_id], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (seen >= 1u) break;
                 __builtin_amdgcn_s_sleep(4);
             }
@@ -429,8 +432,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
         if (threadIdx.x == 0) {
             // ready for the next product; written the way the counters are read and added to (an ordinary store
             // would sit in this XCD's L2, out of sight of the other XCDs' atomics, until the kernel ends)
-            __hip_atomic_store(&dtl_tickets[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&dtl_arrived[tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&dtl_tickets[g.split_slot][tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&dtl_arrived[g.split_slot][tile_id], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 
@@ -898,13 +901,28 @@ inline size_t dtl_pair_split_bytes(long long m, long long n, long long k) {
     return (size_t)(((m + bm - 1) / bm) * ((n + bn - 1) / bn)) * bm * bn * sizeof(float);
 }
 
+// The counter set of a stream (-1: all sets are taken by other streams).
+inline int split_slot_of(hipStream_t st) {
+    static std::mutex mu;
+    static hipStream_t owner[kSplitSlots];
+    static int used = 0;
+    std::lock_guard<std::mutex> lock(mu);
+    for (int i = 0; i < used; i++)
+        if (owner[i] == st) return i;
+    if (used == kSplitSlots) return -1;
+    owner[used] = st;
+    return used++;
+}
+
 template <int CT>
 int launch_dtl(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
     g.splits = 1;
     if (batch == 1 && g.partials) {
         const int c = dtl_pair_split(g.m, g.n, g.k);
-        if (c >= 0 && dtl_pair_split_bytes(g.m, g.n, g.k) <= g.partial_bytes) {
+        const int slot = c >= 0 ? split_slot_of(st) : -1;
+        if (c >= 0 && slot >= 0 && dtl_pair_split_bytes(g.m, g.n, g.k) <= g.partial_bytes) {
             g.splits = 2;
+            g.split_slot = slot;
             if (c == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
             return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
         }

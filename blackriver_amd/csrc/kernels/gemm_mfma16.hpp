@@ -76,6 +76,7 @@ struct GemmArgs {
     int splits = 1;
     float* partials = nullptr;
     size_t partial_bytes = 0;
+    int split_slot = 0;   // which set of the library's arrival counters the two slices of a tile meet through (one per stream)
 };
 
 template <int CT>

@@ -2,6 +2,8 @@
 layout, storage type and compute type, odd sizes, batching, bias, alpha and
 accumulation.  Tolerances: 2e-2 relative for fp16 / bf16 operands, 1e-5 for
 the fp32-operand kernel."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -303,6 +305,48 @@ def test_gemm_staged_split_k(ta, tb, a_dt, b_dt, c_dt):
     assert_close(to_host64(c).reshape(m, n), ref, 2e-2, "split-k staged gemm")
     if c_dt == F32:
         assert np.sqrt(np.mean((to_host64(c).reshape(m, n) - ref) ** 2)) < 1e-3 * np.sqrt(np.mean(ref ** 2))
+
+
+def test_gemm_split_in_two_on_two_streams_at_once():
+    """The 4h -> h shape ([2048 x 4096] from K = 16384, split in two inside
+    the kernel) on two streams at the same time, each with its own operands
+    and workspace: the slices of a tile meet through a counter set per stream,
+    so both streams give the bits they give alone."""
+    torch.manual_seed(5)
+    m, n, k = 2048, 4096, 16384
+    lib = hip.load()
+    need = lib.br_hip_gemm_staged_workspace(0, 1, m, n, k, F16, F16, 1)
+    assert need >= m * n * 4          # room for the partial tiles: this shape takes the split
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    jobs = []
+    for _ in streams:
+        a = torch.randn((m, k), device="cuda").half()
+        b = torch.randn((n, k), device="cuda").half()
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        jobs.append((a, b, ws))
+    torch.cuda.synchronize()
+
+    def launch(job, c, st):
+        a, b, ws = job
+        call("br_hip_gemm_staged", 0, 1, m, n, k, 1.0, ptr(a), F16, k, 0, ptr(b), F16, k, 0, 0, ptr(c), F32, n, 0, None, 1,
+             hip.GEMM_F16, ptr(ws), need, ctypes.c_void_p(st.cuda_stream))
+    alone = []
+    for job, st in zip(jobs, streams):
+        c = torch.full((m, n), float("nan"), device="cuda")
+        launch(job, c, st)
+        torch.cuda.synchronize()
+        alone.append(c)
+    together = [[torch.full((m, n), float("nan"), device="cuda") for _ in range(4)] for _ in streams]
+    torch.cuda.synchronize()
+    for r in range(4):
+        for i, (job, st) in enumerate(zip(jobs, streams)):
+            launch(job, together[i][r], st)
+    torch.cuda.synchronize()
+    for i in range(2):
+        for r in range(4):
+            assert torch.equal(together[i][r], alone[i]), (i, r)
+    ref = jobs[0][0][:64].double() @ jobs[0][1].double().t()
+    assert bool(((alone[0][:64].double() - ref).abs() <= 1e-5 * (ref.abs() + ref.pow(2).mean().sqrt()) * (k ** 0.5)).all())
 
 
 def test_gemm_staged_falls_back():
