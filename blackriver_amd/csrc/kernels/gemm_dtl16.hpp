@@ -344,7 +344,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                 } else {
                     wait_vmem<0>();
                 }
-                // every wave has now read all of tile t, so its buffer can be refilled
+                // every wave has now read all of tile t (__syncthreads waits for the wave's own LDS reads to
+                // complete, lgkmcnt(0), before the barrier), so its buffer can be refilled
                 __syncthreads();
                 if (t + STAGES < nk) issue(t + STAGES);
                 __builtin_amdgcn_sched_barrier(0);
