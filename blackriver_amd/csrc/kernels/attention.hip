@@ -17,7 +17,9 @@
 // log(sum exp) of each score row for the backward pass.
 //
 // Forward kernel.  One workgroup = 4 waves = 128 queries of one (batch, head);
-// each wave owns 32 queries.  Keys / values stream through LDS in tiles of 64;
+// each wave owns 32 queries (launches too small to fill the chip that way take
+// 64-query workgroups whose waves share the keys of a tile, see the kernel).
+// Keys / values stream through LDS in tiles of 64, global memory -> LDS direct;
 // tiles wholly above the diagonal (or at / beyond valid[b]) are skipped, which
 // is exact because their probabilities are exactly zero.  Per tile and wave:
 //   S^T[key, query] = K . Q^T     16 x v_mfma_f32_32x32x16 (A = K rows from
@@ -35,6 +37,7 @@
 // different 64-byte groups (transposing reads).
 #include "common.hpp"
 #include "gemm_mfma16.hpp"
+#include "lds_direct.hpp"
 
 #include <float.h>
 
@@ -50,8 +53,6 @@ constexpr int kChunks = kHD / 8;  // 16-byte chunks per row
 constexpr int kBQ = 128;          // queries per workgroup (forward, dq pass)
 constexpr int kBK = 64;           // keys per LDS tile
 constexpr int kThreads = 256;
-
-typedef __attribute__((address_space(3))) unsigned char lds_byte;
 
 struct FlashArgs {
     const u16* q;
@@ -77,30 +78,43 @@ __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 
 // byte offset of chunk c of row r in a [rows][16 chunks] tile image
 __device__ __forceinline__ unsigned slot(int r, int c) { return (unsigned)((r * kChunks + (c ^ swz(r))) * 16); }
 
-// Cooperative load of ROWS x 128 16-bit elements (rows row0.., clamped to
-// `rows` - 1) into registers, then into an LDS image.  256 threads, 16 bytes
-// each per pass; 16 consecutive threads fetch one contiguous 256-byte row.
-template <int ROWS>
-struct TileLoader {
-    static constexpr int kPasses = ROWS * kChunks / kThreads;
-    u32x4 regs[kPasses];
-    __device__ __forceinline__ void fetch(const u16* base, long long row_stride, int row0, int rows) {
-#pragma unroll
-        for (int i = 0; i < kPasses; i++) {
-            const int idx = threadIdx.x + i * kThreads;
-            int r = row0 + idx / kChunks;
-            r = r < rows ? r : rows - 1;
-            regs[i] = *reinterpret_cast<const u32x4*>(base + (long long)r * row_stride + (idx % kChunks) * 8);
-        }
+// Direct-to-LDS fill of a tile image [64 rows][16 chunks] by the workgroup's four waves: wave w issues the
+// wave-wide loads number w, w + 4, w + 8, w + 12 of the tile, each 1 KiB = 4 image rows; lane l of load L lands in
+// image row 4 L + l / 16 at chunk position l % 16, so it fetches the chunk that `slot` puts there,
+// (l % 16) ^ swz(row) -- and swz(row) = ((l / 16) << 2) | (L & 3), with L & 3 = w for every load of a wave: one
+// per-lane offset serves all four loads, the 16-row blocks differ in the (scalar) base address only.  Rows past the
+// end of the tensor read its last row, as the kernels' masks expect; only a ragged last tile takes that path.
+struct TileFill {
+    unsigned voff;  // this lane's byte offset inside a block of 16 rows
+    unsigned cb;    // ... of which its chunk inside the row
+    int lr;         // its row inside the block
+    __device__ __forceinline__ TileFill(int lane, int wave, long long row_elems) {
+        lr = 4 * wave + (lane >> 4);
+        cb = (unsigned)(((lane & 15) ^ ((lane >> 4) << 2) ^ wave) * 16);
+        voff = (unsigned)lr * (unsigned)(row_elems * 2) + cb;
     }
-    __device__ __forceinline__ void store(unsigned char* tile) const {
+    // rows r0 .. r0 + 63 of `base` (row stride row_elems) into the image at LDS byte address lds_tile
+    __device__ __forceinline__ void fill(unsigned lds_tile, const u16* base, long long row_elems, int r0, int rows,
+                                         int wave) const {
+        const u16* src = base + (long long)r0 * row_elems;
+        if (r0 + kBK <= rows) {
 #pragma unroll
-        for (int i = 0; i < kPasses; i++) {
-            const int idx = threadIdx.x + i * kThreads;
-            *reinterpret_cast<u32x4*>(tile + slot(idx / kChunks, idx % kChunks)) = regs[i];
+            for (int n = 0; n < 4; n++) dtl_load(lds_tile + (4 * n + wave) * 1024, voff, src + 16 * n * row_elems);
+        } else {
+#pragma unroll
+            for (int n = 0; n < 4; n++) {
+                int r = 16 * n + lr;
+                r = r < rows - r0 ? r : rows - 1 - r0;
+                dtl_load(lds_tile + (4 * n + wave) * 1024, (unsigned)r * (unsigned)(row_elems * 2) + cb, src);
+            }
         }
     }
 };
+// 64 floats src[r0 .. r0 + 63] (clamped to src[rows - 1]) to LDS byte address lds_row; one wave-wide load
+__device__ __forceinline__ void fill_row(unsigned lds_row, const float* src, int r0, int rows, int lane) {
+    const int r = lane < rows - r0 ? lane : rows - 1 - r0;
+    dtl_load_dword(lds_row, (unsigned)r * 4u, src + r0);
+}
 
 // MFMA operand fragments of a tile image.  Every lane-dependent part of an
 // address is computed once (constructor); inside the tile loops a read is that
@@ -115,17 +129,18 @@ struct TileLoader {
 struct FragOffsets {
     unsigned rows[8];
     unsigned cols_lo[4], cols_hi[4];
-    __device__ __forceinline__ explicit FragOffsets(int lane) {
+    // row_bias (a multiple of 16): tile rows are counted from there, for a wave that owns part of every tile
+    __device__ __forceinline__ explicit FragOffsets(int lane, int row_bias = 0) {
         const int i = lane & 15, half = lane >> 5;
 #pragma unroll
-        for (int ks = 0; ks < 8; ks++) rows[ks] = slot(lane & 31, ks * 2 + half);
+        for (int ks = 0; ks < 8; ks++) rows[ks] = slot(lane & 31, ks * 2 + half) + row_bias * 256;
 #pragma unroll
         for (int db = 0; db < 4; db++) {
             // a group of 16 lanes reads 4 tile rows (i >> 2) x 16 d; lane i receives d column i
             const int d = db * 32 + ((lane >> 4) & 1) * 16 + (i & 3) * 4;
             const int ja = half * 4 + (i >> 2);
-            cols_lo[db] = slot(ja, d >> 3) + (d & 7) * 2;
-            cols_hi[db] = slot(ja + 8, d >> 3) + (d & 7) * 2;
+            cols_lo[db] = slot(ja, d >> 3) + (d & 7) * 2 + row_bias * 256;
+            cols_hi[db] = slot(ja + 8, d >> 3) + (d & 7) * 2 + row_bias * 256;
         }
     }
     // rows r0 .. r0 + 31 (r0 a multiple of 32) of the tile at byte offset `tile`
@@ -172,40 +187,31 @@ __device__ __forceinline__ float score(float dot, float scale, float bias, int q
 constexpr int kTileBytes = kBK * kHD * 2;
 constexpr int kStageBytes = 2 * kTileBytes + kBK * 4;
 
-// Register staging of one stage (global -> registers -> LDS), so that the
-// loads of tile t+1 are in flight while tile t is computed.
-struct StageLoader {
-    TileLoader<kBK> k, v;
-    float bias;
-    __device__ __forceinline__ void fetch(const u16* kbase, const u16* vbase, const float* alibi_row, long long row,
-                                          int k0, int tokens) {
-        k.fetch(kbase, row, k0, tokens);
-        v.fetch(vbase, row, k0, tokens);
-        if (threadIdx.x < kBK) {
-            const int key = k0 + (int)threadIdx.x;
-            bias = alibi_row[key < tokens ? key : tokens - 1];
-        }
-    }
-    __device__ __forceinline__ void store(unsigned char* stage) const {
-        k.store(stage);
-        v.store(stage + kTileBytes);
-        if (threadIdx.x < kBK) reinterpret_cast<float*>(stage + 2 * kTileBytes)[threadIdx.x] = bias;
-    }
-};
-
-template <int CT>
-__global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
+// (G, KH) = (4, 1): four waves, each with 32 queries and every key of a tile; 128 queries per workgroup.
+// (G, KH) = (2, 2): 64 queries per workgroup; wave (qg, kh) has the queries of group qg = wave % 2 and keys
+// 32 * kh .. + 31 of every tile, with its own running maximum, sum and context; the two halves of a query group are
+// merged through LDS at the end (the usual rescaling of two partial softmax sums).  Twice the workgroups, half the
+// work per wave and tile: for launches whose 128-query workgroups would leave compute units empty (one sequence of
+// 512 tokens and 32 heads: 128 of them), where a workgroup's walk over its key tiles is the whole kernel time.
+template <int CT, int G, int KH>
+__global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_fwd_kernel(FlashArgs a) {
+    static_assert(G * KH == 4, "TileFill deals a tile to four waves");
+    constexpr int BQ = 32 * G;         // queries per workgroup
+    constexpr int NKB = 2 / KH;        // 32-key blocks of a tile per wave
+    constexpr int kSpan = kBK / KH;    // keys of a tile per wave
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
+    static_assert(KH == 1 || 2 * kStageBytes >= G * (64 * 64 + 2 * 64) * 4, "the merge puts G contexts of 64 x 64 floats, their m and l into the stages");
     const int lane = threadIdx.x & 63, half = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: branches on it are scalar
+    const int qg = KH == 1 ? wave : wave % G, kh = KH == 1 ? 0 : wave / G;
     // workgroups are numbered longest first: the query tiles with the most
     // visible keys of every (batch, head), then the next ones, ...
-    const int tiles_q = (a.tokens + kBQ - 1) / kBQ;
+    const int tiles_q = (a.tokens + BQ - 1) / BQ;
     const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
     const int qt = tiles_q - 1 - (int)(blockIdx.x / a.batch_heads);
     const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
     const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
-    const int q0 = qt * kBQ + wave * 32;
+    const int q0 = qt * BQ + qg * 32;
     const int query = q0 + (lane & 31);
     const int qrow = query < a.tokens ? query : a.tokens - 1;
     const float* alibi_row = a.alibi + (long long)h * a.tokens;
@@ -222,39 +228,49 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
         for (int v = 0; v < 16; v++) o[db][v] = 0.f;
     float m = -INFINITY, l = 0.f;
 
-    const int nkeys = visible_keys(qt * kBQ + kBQ, valid, a.tokens);
+    const int nkeys = visible_keys(qt * BQ + BQ, valid, a.tokens);
     const int ntiles = (nkeys + kBK - 1) / kBK;
     // keys this wave's queries can see (a wave may idle through the last tiles)
     const int wave_keys = visible_keys(q0 + 32, valid, a.tokens);
 
-    const FragOffsets fo(lane);
+    const FragOffsets fo(lane, kh * 32);
     const lds_byte* ldsb = (const lds_byte*)lds;
-    StageLoader ld;
-    ld.fetch(a.k + base, a.v + base, alibi_row, a.row, 0, a.tokens);
-    ld.store(lds);
-    if (ntiles > 1) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, kBK, a.tokens);
+    // Key tile t goes straight from global memory into stage t % 2 (K image, V image, the tile's ALiBi row): issued
+    // at the start of step t - 1, when the barrier that ended step t - 2 has freed the stage, and waited for at the
+    // end of step t - 1.  Every wave issues its quarter of the images and waits for its own loads before the barrier.
+    const unsigned lds0 = (unsigned)(unsigned long long)ldsb;
+    const TileFill kv_fill(lane, wave, a.row);
+    auto issue = [&](int t, unsigned stage_bytes) {
+        const unsigned st = lds0 + stage_bytes;
+        kv_fill.fill(st, a.k + base, a.row, t * kBK, a.tokens, wave);
+        kv_fill.fill(st + kTileBytes, a.v + base, a.row, t * kBK, a.tokens, wave);
+        fill_row(st + 2 * kTileBytes, alibi_row, t * kBK, a.tokens, lane);
+    };
+    issue(0, 0);
+    wait_vmem<0>();
     __syncthreads();
     // one key tile; the stage is a compile-time constant so that every LDS
     // address is a per-lane offset computed once plus an immediate
     auto tile_step = [&](auto stage_c, int t) {
         constexpr int kStage = decltype(stage_c)::value * kStageBytes;
-        const int k0 = t * kBK;
+        const int k0 = t * kBK + kh * 32;   // this wave's first key of the tile
+        if (t + 1 < ntiles) issue(t + 1, kStageBytes - kStage);
         if (k0 < wave_keys) {
-            f32x16 s[2];
+            f32x16 s[NKB];
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
                 for (int v = 0; v < 16; v++) s[kb][v] = 0.f;
 #pragma unroll
                 for (int ks = 0; ks < 8; ks++)
                     s[kb] = Cvt<CT>::mfma(fo.frag_rows(ldsb, kStage, kb * 32, ks), qf[ks], s[kb]);
             }
-            const float* tb = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + half * 4;
+            const float* tb = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + kh * 32 + half * 4;
             float mt = -INFINITY;
-            // tiles wholly below the diagonal and inside the sequence need no mask
-            if (k0 + kBK - 1 <= q0 && k0 + kBK <= valid) {
+            // keys wholly below the diagonal and inside the sequence need no mask
+            if (k0 + kSpan - 1 <= q0 && k0 + kSpan <= valid) {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const float4 bv = *reinterpret_cast<const float4*>(tb + kb * 32 + g * 8);
@@ -269,7 +285,7 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
                     }
             } else {
 #pragma unroll
-                for (int kb = 0; kb < 2; kb++)
+                for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const float4 bv = *reinterpret_cast<const float4*>(tb + kb * 32 + g * 8);
@@ -288,7 +304,7 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
             const float alpha = __expf(m - m_new);
             float sum = 0.f;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
+            for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) {
                     const float p = __expf(s[kb][v] - m_new);
@@ -298,33 +314,59 @@ __global__ __launch_bounds__(kThreads, 2) void flash_fwd_kernel(FlashArgs a) {
             sum += xor32(sum);
             l = l * alpha + sum;
             m = m_new;
+            u32x4 pf[2 * NKB];
+#pragma unroll
+            for (int j = 0; j < 2 * NKB; j++) {
+                const int kb = j >> 1, vb = (j & 1) * 8;
+                float p8[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) p8[e] = s[kb][vb + e];
+                pf[j] = pack8<CT>(p8);
+            }
 #pragma unroll
             for (int db = 0; db < 4; db++)
 #pragma unroll
                 for (int v = 0; v < 16; v++) o[db][v] *= alpha;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int kb = j >> 1, vb = (j & 1) * 8;
-                float p8[8];
-#pragma unroll
-                for (int e = 0; e < 8; e++) p8[e] = s[kb][vb + e];
-                const u32x4 pf = pack8<CT>(p8);
+            for (int j = 0; j < 2 * NKB; j++)
 #pragma unroll
                 for (int db = 0; db < 4; db++)
-                    o[db] = Cvt<CT>::mfma(fo.frag_cols(ldsb, kStage + kTileBytes, db, kb * 32 + (j & 1) * 16), pf, o[db]);
-            }
+                    o[db] = Cvt<CT>::mfma(fo.frag_cols(ldsb, kStage + kTileBytes, db, (j >> 1) * 32 + (j & 1) * 16), pf[j], o[db]);
         }
-        // tile t+1 (in registers since the previous step) goes into the other
-        // stage, whose last readers passed the barrier of step t-1
-        if (t + 1 < ntiles) {
-            ld.store(lds + (kStageBytes - kStage));
-            if (t + 2 < ntiles) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, k0 + 2 * kBK, a.tokens);
-        }
+        wait_vmem<0>();   // this wave's part of tile t + 1 is in
         __syncthreads();
     };
     for (int t = 0; t < ntiles; t += 2) {
         tile_step(std::integral_constant<int, 0>(), t);
         if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
+    }
+
+    if (KH == 2) {
+        // Merge the two key halves of each query group: the waves with the odd halves leave m, l and their context
+        // in LDS (every wave is past the loop's last barrier: the stages are free), the others rescale both to the
+        // common maximum.  A half that met no key has m = -inf, l = 0 and weighs nothing; key 0 is in the even half
+        // and visible to every query of a non-empty sequence, so the common maximum is never -inf.
+        float* const xo = reinterpret_cast<float*>(lds) + qg * (64 * 64);
+        float* const xml = reinterpret_cast<float*>(lds) + G * 64 * 64 + qg * 128;
+        if (kh == 1) {
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) xo[(db * 16 + v) * 64 + lane] = o[db][v];
+            xml[lane] = m;
+            xml[64 + lane] = l;
+        }
+        __syncthreads();
+        if (kh == 1) return;
+        const float m1 = xml[lane], l1 = xml[64 + lane];
+        const float m_all = fmaxf(m, m1);
+        const float w0 = __expf(m - m_all), w1 = __expf(m1 - m_all);
+        l = l * w0 + l1 * w1;
+        m = m_all;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) o[db][v] = o[db][v] * w0 + xo[(db * 16 + v) * 64 + lane] * w1;
     }
 
     if (query < a.tokens) {
@@ -355,25 +397,6 @@ __device__ __forceinline__ float to_f32<BR_GEMM_BF16>(u16 x) { return __uint_as_
 // the tile's lse and delta values.
 constexpr int kQStageBytes = 2 * kTileBytes + 2 * kBK * 4;
 
-struct QStageLoader {
-    TileLoader<kBK> q, g;
-    float stat;
-    __device__ __forceinline__ void fetch(const FlashArgs& a, long long base, long long obase, int bh, int q0) {
-        q.fetch(a.q + base, a.row, q0, a.tokens);
-        g.fetch(a.d_o + obase, a.orow, q0, a.tokens);
-        if (threadIdx.x < 2 * kBK) {
-            const int t = q0 + (int)(threadIdx.x & (kBK - 1));
-            const float* src = threadIdx.x < kBK ? a.lse : a.delta;
-            stat = src[(long long)bh * a.tokens + (t < a.tokens ? t : a.tokens - 1)];
-        }
-    }
-    __device__ __forceinline__ void store(unsigned char* stage) const {
-        q.store(stage);
-        g.store(stage + kTileBytes);
-        if (threadIdx.x < 2 * kBK) reinterpret_cast<float*>(stage + 2 * kTileBytes)[threadIdx.x] = stat;
-    }
-};
-
 // dK, dV of 128 keys (32 per wave) of one (batch, head): queries stream through
 // LDS in tiles of 64.  Per wave and 32-query block:
 //   S[query, key]  = Q . K^T        (A = Q rows from LDS, B = K in registers)
@@ -381,17 +404,26 @@ struct QStageLoader {
 //   P = exp(score - lse),  dS = P o (dP - delta)
 //   dV[key, d] += P^T . dO,  dK[key, d] += dS^T . Q   (A from the accumulators,
 //                                    B by transposing reads of the same tiles)
-template <int CT>
-__global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
+// (G, QH) = (4, 1): 128 keys per workgroup, 32 per wave, every query of a tile.  (2, 2): 64 keys per workgroup; wave
+// (kg, qh) has the keys of group kg = wave % 2 and queries 32 * qh .. + 31 of every query tile; the two partial dK
+// and dV of a key group are added through LDS at the end.
+template <int CT, int G, int QH>
+__global__ __launch_bounds__(64 * G * QH) void flash_bwd_dkv_kernel(FlashArgs a) {
+    static_assert(G * QH == 4, "TileFill deals a tile to four waves");
+    constexpr int BKEYS = 32 * G;      // keys per workgroup
+    constexpr int NQB = 2 / QH;        // 32-query blocks of a tile per wave
+    constexpr int kSpan = kBK / QH;    // queries of a tile per wave
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kQStageBytes];
+    static_assert(2 * kQStageBytes >= G * 64 * 64 * 4, "the merge puts G blocks of 64 x 64 floats into the stages");
     const int lane = threadIdx.x & 63, half = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: branches on it are scalar
+    const int kg = QH == 1 ? wave : wave % G, qh = QH == 1 ? 0 : wave / G;
     const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
     const int kt = (int)(blockIdx.x / a.batch_heads);  // key tile 0 meets the most queries: longest first
     const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
     const long long obase = (long long)b * a.obatch + (long long)h * a.head;
     const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
-    const int key0 = kt * kBQ + wave * 32;
+    const int key0 = kt * BKEYS + kg * 32;
     const int key = key0 + (lane & 31);
     const int krow = key < a.tokens ? key : a.tokens - 1;
     const float bias = a.alibi[(long long)h * a.tokens + krow];
@@ -412,30 +444,39 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
     // queries that can see any key of this workgroup start at its first key
     // (none at all when the keys lie in the padding); an empty sequence has
     // uniform probabilities everywhere, so nothing is skipped for it
-    const bool dead_group = valid > 0 && kt * kBQ >= valid;
-    const int q_begin = valid > 0 ? (kt * kBQ / kBK) * kBK : 0;
+    const bool dead_group = valid > 0 && kt * BKEYS >= valid;
+    const int q_begin = valid > 0 ? (kt * BKEYS / kBK) * kBK : 0;
     const int ntiles = dead_group ? 0 : (a.tokens - q_begin + kBK - 1) / kBK;
     const bool dead_wave = valid > 0 && key0 >= valid;
 
-    const FragOffsets fo(lane);
+    const FragOffsets fo(lane, qh * 32);
     const lds_byte* ldsb = (const lds_byte*)lds;
-    QStageLoader ld;
-    if (ntiles > 0) {
-        ld.fetch(a, base, obase, bh, q_begin);
-        ld.store(lds);
-        if (ntiles > 1) ld.fetch(a, base, obase, bh, q_begin + kBK);
-    }
+    // query tile t (Q image, dO image, the tile's lse and delta rows) goes straight into stage t % 2, as the key
+    // tiles of the forward kernel do
+    const unsigned lds0 = (unsigned)(unsigned long long)ldsb;
+    const TileFill q_fill(lane, wave, a.row), g_fill(lane, wave, a.orow);
+    auto issue = [&](int t, unsigned stage_bytes) {
+        const unsigned st = lds0 + stage_bytes;
+        const int r0 = q_begin + t * kBK;
+        q_fill.fill(st, a.q + base, a.row, r0, a.tokens, wave);
+        g_fill.fill(st + kTileBytes, a.d_o + obase, a.orow, r0, a.tokens, wave);
+        fill_row(st + 2 * kTileBytes, a.lse + (long long)bh * a.tokens, r0, a.tokens, lane);
+        fill_row(st + 2 * kTileBytes + kBK * 4, a.delta + (long long)bh * a.tokens, r0, a.tokens, lane);
+    };
+    if (ntiles > 0) issue(0, 0);
+    wait_vmem<0>();
     __syncthreads();
     auto tile_step = [&](auto stage_c, int t) {
         constexpr int kStage = decltype(stage_c)::value * kQStageBytes;
-        const int q0 = q_begin + t * kBK;
-        const float* tl = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + half * 4;
+        const int q0 = q_begin + t * kBK + qh * 32;   // this wave's first query of the tile
+        if (t + 1 < ntiles) issue(t + 1, kQStageBytes - kStage);
+        const float* tl = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + qh * 32 + half * 4;
         const float* td = tl + kBK;
-        // a tile whose queries all precede this wave's keys sees none of them
-        if (!dead_wave && !(valid > 0 && q0 + kBK - 1 < key0)) {
-            const bool open = q0 >= key0 + 31 && key0 + 32 <= valid && q0 + kBK <= a.tokens;
+        // queries that all precede this wave's keys see none of them
+        if (!dead_wave && !(valid > 0 && q0 + kSpan - 1 < key0)) {
+            const bool open = q0 >= key0 + 31 && key0 + 32 <= valid && q0 + kSpan <= a.tokens;
 #pragma unroll
-            for (int qb = 0; qb < 2; qb++) {
+            for (int qb = 0; qb < NQB; qb++) {
                 f32x16 s, dp;
 #pragma unroll
                 for (int v = 0; v < 16; v++) s[v] = dp[v] = 0.f;
@@ -493,15 +534,44 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
                 }
             }
         }
-        if (t + 1 < ntiles) {
-            ld.store(lds + (kQStageBytes - kStage));
-            if (t + 2 < ntiles) ld.fetch(a, base, obase, bh, q0 + 2 * kBK);
-        }
+        wait_vmem<0>();   // this wave's part of tile t + 1 is in
         __syncthreads();
     };
     for (int t = 0; t < ntiles; t += 2) {
         tile_step(std::integral_constant<int, 0>(), t);
         if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
+    }
+
+    if (QH == 2) {
+        // the waves with the odd query halves hand their sums over, dK first, then dV (every wave is past the loop's
+        // last barrier: the stages are free)
+        float* const x = reinterpret_cast<float*>(lds) + kg * (64 * 64);
+        if (qh == 1) {
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) x[(db * 16 + v) * 64 + lane] = dk[db][v];
+        }
+        __syncthreads();
+        if (qh == 0) {
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) dk[db][v] += x[(db * 16 + v) * 64 + lane];
+        }
+        __syncthreads();
+        if (qh == 1) {
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) x[(db * 16 + v) * 64 + lane] = dv[db][v];
+        }
+        __syncthreads();
+        if (qh == 1) return;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) dv[db][v] += x[(db * 16 + v) * 64 + lane];
     }
 
     // accumulator element v of block db: key key0 + acc_row(v), d = 32 * db + lane % 32
@@ -527,17 +597,25 @@ __global__ __launch_bounds__(kThreads) void flash_bwd_dkv_kernel(FlashArgs a) {
 // dQ of 128 queries (32 per wave) of one (batch, head): the forward's loop over
 // key tiles, with  S^T = K . Q^T,  dP^T = V . dO^T  and
 // dQ^T[d, query] += K^T . dS^T  (K^T by transposing reads of the K tile).
-template <int CT>
-__global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) {
+// (G, KH) = (2, 2): 64 queries per workgroup, the keys of every tile split between two waves as in the forward
+// kernel; the two partial dQ of a query group are added through LDS at the end.
+template <int CT, int G, int KH>
+__global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_bwd_dq_kernel(FlashArgs a) {
+    static_assert(G * KH == 4, "TileFill deals a tile to four waves");
+    constexpr int BQ = 32 * G;
+    constexpr int NKB = 2 / KH;
+    constexpr int kSpan = kBK / KH;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * kStageBytes];
+    static_assert(2 * kStageBytes >= G * 64 * 64 * 4, "the merge puts G blocks of 64 x 64 floats into the stages");
     const int lane = threadIdx.x & 63, half = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: branches on it are scalar
-    const int tiles_q = (a.tokens + kBQ - 1) / kBQ;
+    const int qg = KH == 1 ? wave : wave % G, kh = KH == 1 ? 0 : wave / G;
+    const int tiles_q = (a.tokens + BQ - 1) / BQ;
     const int bh = (int)(blockIdx.x % a.batch_heads), b = bh / a.heads, h = bh % a.heads;
     const int qt = tiles_q - 1 - (int)(blockIdx.x / a.batch_heads);
     const long long base = (long long)b * a.batch_stride + (long long)h * a.head;
     const int valid = a.valid[b] < a.tokens ? a.valid[b] : a.tokens;
-    const int q0 = qt * kBQ + wave * 32;
+    const int q0 = qt * BQ + qg * 32;
     const int query = q0 + (lane & 31);
     const int qrow = query < a.tokens ? query : a.tokens - 1;
     const float* alibi_row = a.alibi + (long long)h * a.tokens;
@@ -561,7 +639,7 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
         }
     }
     delta += __shfl_xor(delta, 32, kWave);
-    if (half == 0 && query < a.tokens) a.delta[(long long)bh * a.tokens + query] = delta;
+    if (half == 0 && kh == 0 && query < a.tokens) a.delta[(long long)bh * a.tokens + query] = delta;
 #pragma unroll
     for (int ks = 0; ks < 8; ks++)
         qf[ks] = *reinterpret_cast<const u32x4*>(a.q + base + (long long)qrow * a.row + ks * 16 + half * 8);
@@ -571,25 +649,35 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
 #pragma unroll
         for (int v = 0; v < 16; v++) dq[db][v] = 0.f;
 
-    const int nkeys = visible_keys(qt * kBQ + kBQ, valid, a.tokens);
+    const int nkeys = visible_keys(qt * BQ + BQ, valid, a.tokens);
     const int ntiles = (nkeys + kBK - 1) / kBK;
     const int wave_keys = visible_keys(q0 + 32, valid, a.tokens);
 
-    const FragOffsets fo(lane);
+    const FragOffsets fo(lane, kh * 32);
     const lds_byte* ldsb = (const lds_byte*)lds;
-    StageLoader ld;
-    ld.fetch(a.k + base, a.v + base, alibi_row, a.row, 0, a.tokens);
-    ld.store(lds);
-    if (ntiles > 1) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, kBK, a.tokens);
+    // Key tile t goes straight from global memory into stage t % 2 (K image, V image, the tile's ALiBi row): issued
+    // at the start of step t - 1, when the barrier that ended step t - 2 has freed the stage, and waited for at the
+    // end of step t - 1.  Every wave issues its quarter of the images and waits for its own loads before the barrier.
+    const unsigned lds0 = (unsigned)(unsigned long long)ldsb;
+    const TileFill kv_fill(lane, wave, a.row);
+    auto issue = [&](int t, unsigned stage_bytes) {
+        const unsigned st = lds0 + stage_bytes;
+        kv_fill.fill(st, a.k + base, a.row, t * kBK, a.tokens, wave);
+        kv_fill.fill(st + kTileBytes, a.v + base, a.row, t * kBK, a.tokens, wave);
+        fill_row(st + 2 * kTileBytes, alibi_row, t * kBK, a.tokens, lane);
+    };
+    issue(0, 0);
+    wait_vmem<0>();
     __syncthreads();
     auto tile_step = [&](auto stage_c, int t) {
         constexpr int kStage = decltype(stage_c)::value * kStageBytes;
-        const int k0 = t * kBK;
-        const float* tb = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + half * 4;
+        const int k0 = t * kBK + kh * 32;   // this wave's first key of the tile
+        if (t + 1 < ntiles) issue(t + 1, kStageBytes - kStage);
+        const float* tb = reinterpret_cast<const float*>(lds + kStage + 2 * kTileBytes) + kh * 32 + half * 4;
         if (k0 < wave_keys) {
-            const bool open = k0 + kBK - 1 <= q0 && k0 + kBK <= valid;
+            const bool open = k0 + kSpan - 1 <= q0 && k0 + kSpan <= valid;
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < NKB; kb++) {
                 f32x16 s, dp;
 #pragma unroll
                 for (int v = 0; v < 16; v++) s[v] = dp[v] = 0.f;
@@ -637,15 +725,28 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
                 }
             }
         }
-        if (t + 1 < ntiles) {
-            ld.store(lds + (kStageBytes - kStage));
-            if (t + 2 < ntiles) ld.fetch(a.k + base, a.v + base, alibi_row, a.row, k0 + 2 * kBK, a.tokens);
-        }
+        wait_vmem<0>();   // this wave's part of tile t + 1 is in
         __syncthreads();
     };
     for (int t = 0; t < ntiles; t += 2) {
         tile_step(std::integral_constant<int, 0>(), t);
         if (t + 1 < ntiles) tile_step(std::integral_constant<int, 1>(), t + 1);
+    }
+
+    if (KH == 2) {
+        float* const x = reinterpret_cast<float*>(lds) + qg * (64 * 64);
+        if (kh == 1) {
+#pragma unroll
+            for (int db = 0; db < 4; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) x[(db * 16 + v) * 64 + lane] = dq[db][v];
+        }
+        __syncthreads();
+        if (kh == 1) return;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) dq[db][v] += x[(db * 16 + v) * 64 + lane];
     }
 
     if (query < a.tokens && !a.grad16) {
@@ -672,10 +773,22 @@ __global__ __launch_bounds__(kThreads, 2) void flash_bwd_dq_kernel(FlashArgs a) 
     }
 }
 
+// Whether a launch that would take `workgroups` workgroups of 128 queries (or keys) runs on twice as many of 64
+// instead, each tile's work split between two waves: where the wider ones would leave compute units empty.
+#ifndef BR_FA_SPLIT_BELOW
+#define BR_FA_SPLIT_BELOW 256
+#endif
+#ifndef BR_FA_DKV_SPLIT_BELOW
+#define BR_FA_DKV_SPLIT_BELOW 256
+#endif
+inline bool narrow_split(unsigned workgroups) { return workgroups < (unsigned)BR_FA_SPLIT_BELOW; }
+inline bool narrow_split_dkv(unsigned workgroups) { return workgroups < (unsigned)BR_FA_DKV_SPLIT_BELOW; }
+
 bool flash_shape_ok(int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim, int64_t row, int64_t head,
                     int64_t batch_stride, int64_t orow, int64_t obatch) {
     return batch > 0 && heads > 0 && tokens >= 1 && head_dim == kHD && row % 8 == 0 &&
-           head % 8 == 0 && batch_stride % 8 == 0 && orow % 8 == 0 && obatch % 8 == 0 && batch * heads <= (1 << 20) && tokens <= (1 << 20);
+           head % 8 == 0 && batch_stride % 8 == 0 && orow % 8 == 0 && obatch % 8 == 0 && batch * heads <= (1 << 20) && tokens <= (1 << 20) &&
+           row < (1 << 24) && orow < (1 << 24);   // 64 rows of a tile within a 32-bit byte offset
 }
 
 }  // namespace
@@ -713,10 +826,18 @@ int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype
     a.batch_heads = (int)(batch * heads);
     a.scale = (float)(1.0 / sqrt((double)head_dim));
     const unsigned grid = (unsigned)(((tokens + kBQ - 1) / kBQ) * batch * heads);
-    if (dtype == BR_F16)
-        flash_fwd_kernel<BR_GEMM_F16><<<grid, kThreads, 0, as_stream(stream)>>>(a);
-    else
-        flash_fwd_kernel<BR_GEMM_BF16><<<grid, kThreads, 0, as_stream(stream)>>>(a);
+    if (narrow_split(grid)) {
+        const unsigned grid2 = (unsigned)(((tokens + 63) / 64) * batch * heads);
+        if (dtype == BR_F16)
+            flash_fwd_kernel<BR_GEMM_F16, 2, 2><<<grid2, kThreads, 0, as_stream(stream)>>>(a);
+        else
+            flash_fwd_kernel<BR_GEMM_BF16, 2, 2><<<grid2, kThreads, 0, as_stream(stream)>>>(a);
+    } else {
+        if (dtype == BR_F16)
+            flash_fwd_kernel<BR_GEMM_F16, 4, 1><<<grid, kThreads, 0, as_stream(stream)>>>(a);
+        else
+            flash_fwd_kernel<BR_GEMM_BF16, 4, 1><<<grid, kThreads, 0, as_stream(stream)>>>(a);
+    }
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
 }
@@ -767,12 +888,18 @@ int br_hip_flash_attn_bwd(const void* q, const void* k, const void* v, const voi
     hipStream_t st = as_stream(stream);
     const unsigned tiles = (unsigned)(((tokens + kBQ - 1) / kBQ) * batch * heads);
     // the dQ pass first: it leaves delta behind for the dK / dV pass
+    const unsigned tiles2 = (unsigned)(((tokens + 63) / 64) * batch * heads);
+    const bool split_q = narrow_split(tiles), split_kv = narrow_split_dkv(tiles);
     if (dtype == BR_F16) {
-        flash_bwd_dq_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
-        flash_bwd_dkv_kernel<BR_GEMM_F16><<<tiles, kThreads, 0, st>>>(a);
+        if (split_q) flash_bwd_dq_kernel<BR_GEMM_F16, 2, 2><<<tiles2, kThreads, 0, st>>>(a);
+        else flash_bwd_dq_kernel<BR_GEMM_F16, 4, 1><<<tiles, kThreads, 0, st>>>(a);
+        if (split_kv) flash_bwd_dkv_kernel<BR_GEMM_F16, 2, 2><<<tiles2, kThreads, 0, st>>>(a);
+        else flash_bwd_dkv_kernel<BR_GEMM_F16, 4, 1><<<tiles, kThreads, 0, st>>>(a);
     } else {
-        flash_bwd_dq_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
-        flash_bwd_dkv_kernel<BR_GEMM_BF16><<<tiles, kThreads, 0, st>>>(a);
+        if (split_q) flash_bwd_dq_kernel<BR_GEMM_BF16, 2, 2><<<tiles2, kThreads, 0, st>>>(a);
+        else flash_bwd_dq_kernel<BR_GEMM_BF16, 4, 1><<<tiles, kThreads, 0, st>>>(a);
+        if (split_kv) flash_bwd_dkv_kernel<BR_GEMM_BF16, 2, 2><<<tiles2, kThreads, 0, st>>>(a);
+        else flash_bwd_dkv_kernel<BR_GEMM_BF16, 4, 1><<<tiles, kThreads, 0, st>>>(a);
     }
     BR_HIP_LAUNCH_CHECK();
     return BR_OK;
