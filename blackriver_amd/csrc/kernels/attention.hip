@@ -157,6 +157,12 @@ struct FragOffsets {
     }
 };
 
+// Makes the compiler finish the global loads behind `x` here: it places its own s_waitcnt vmcnt in front of a load's
+// first use, and a first use inside the tile loop would sit behind the direct-to-LDS loads issued at the top of the
+// step (which the compiler does not count) -- the wave would wait for the NEXT tile in the middle of this one.
+template <typename T>
+__device__ __forceinline__ void landed(T& x) { asm volatile("" : "+v"(x)); }
+
 // Row index (within a 32-row accumulator block) of accumulator element v.
 __device__ __forceinline__ int acc_row(int v, int lane) { return (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3); }
 
@@ -246,6 +252,8 @@ __global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_fwd_kernel
         kv_fill.fill(st + kTileBytes, a.v + base, a.row, t * kBK, a.tokens, wave);
         fill_row(st + 2 * kTileBytes, alibi_row, t * kBK, a.tokens, lane);
     };
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) landed(qf[ks]);
     issue(0, 0);
     wait_vmem<0>();
     __syncthreads();
@@ -426,7 +434,7 @@ __global__ __launch_bounds__(64 * G * QH) void flash_bwd_dkv_kernel(FlashArgs a)
     const int key0 = kt * BKEYS + kg * 32;
     const int key = key0 + (lane & 31);
     const int krow = key < a.tokens ? key : a.tokens - 1;
-    const float bias = a.alibi[(long long)h * a.tokens + krow];
+    float bias = a.alibi[(long long)h * a.tokens + krow];
     const float uniform = 1.0f / (float)a.tokens;
 
     u32x4 kf[8], vf[8];
@@ -463,6 +471,12 @@ __global__ __launch_bounds__(64 * G * QH) void flash_bwd_dkv_kernel(FlashArgs a)
         fill_row(st + 2 * kTileBytes, a.lse + (long long)bh * a.tokens, r0, a.tokens, lane);
         fill_row(st + 2 * kTileBytes + kBK * 4, a.delta + (long long)bh * a.tokens, r0, a.tokens, lane);
     };
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+        landed(kf[ks]);
+        landed(vf[ks]);
+    }
+    landed(bias);
     if (ntiles > 0) issue(0, 0);
     wait_vmem<0>();
     __syncthreads();
@@ -619,7 +633,7 @@ __global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_bwd_dq_ker
     const int query = q0 + (lane & 31);
     const int qrow = query < a.tokens ? query : a.tokens - 1;
     const float* alibi_row = a.alibi + (long long)h * a.tokens;
-    const float lse = a.lse[(long long)bh * a.tokens + qrow];
+    float lse = a.lse[(long long)bh * a.tokens + qrow];
     const float uniform = 1.0f / (float)a.tokens;
 
     // The query's dO fragments, and on the way delta[query] = sum_d dO[query, d] * O[query, d]: the two halves of a
@@ -666,6 +680,12 @@ __global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_bwd_dq_ker
         kv_fill.fill(st + kTileBytes, a.v + base, a.row, t * kBK, a.tokens, wave);
         fill_row(st + 2 * kTileBytes, alibi_row, t * kBK, a.tokens, lane);
     };
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+        landed(qf[ks]);
+        landed(gf[ks]);
+    }
+    landed(lse);
     issue(0, 0);
     wait_vmem<0>();
     __syncthreads();
