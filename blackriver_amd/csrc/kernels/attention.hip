@@ -200,7 +200,7 @@ constexpr int kStageBytes = 2 * kTileBytes + kBK * 4;
 // work per wave and tile: for launches whose 128-query workgroups would leave compute units empty (one sequence of
 // 512 tokens and 32 heads: 128 of them), where a workgroup's walk over its key tiles is the whole kernel time.
 template <int CT, int G, int KH>
-__global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_fwd_kernel(FlashArgs a) {
+__global__ __launch_bounds__(64 * G * KH, 2) void flash_fwd_kernel(FlashArgs a) {
     static_assert(G * KH == 4, "TileFill deals a tile to four waves");
     constexpr int BQ = 32 * G;         // queries per workgroup
     constexpr int NKB = 2 / KH;        // 32-key blocks of a tile per wave
@@ -614,7 +614,7 @@ __global__ __launch_bounds__(64 * G * QH) void flash_bwd_dkv_kernel(FlashArgs a)
 // (G, KH) = (2, 2): 64 queries per workgroup, the keys of every tile split between two waves as in the forward
 // kernel; the two partial dQ of a query group are added through LDS at the end.
 template <int CT, int G, int KH>
-__global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_bwd_dq_kernel(FlashArgs a) {
+__global__ __launch_bounds__(64 * G * KH, 2) void flash_bwd_dq_kernel(FlashArgs a) {
     static_assert(G * KH == 4, "TileFill deals a tile to four waves");
     constexpr int BQ = 32 * G;
     constexpr int NKB = 2 / KH;
@@ -794,14 +794,18 @@ __global__ __launch_bounds__(64 * G * KH, KH == 1 ? 2 : 1) void flash_bwd_dq_ker
 }
 
 // Whether a launch that would take `workgroups` workgroups of 128 queries (or keys) runs on twice as many of 64
-// instead, each tile's work split between two waves: where the wider ones would leave compute units empty.
-#ifndef BR_FA_SPLIT_BELOW
-#define BR_FA_SPLIT_BELOW 256
+// instead, each tile's work split between two waves: where the wider ones would leave compute units empty or with
+// one workgroup each.  Measured at 32 heads x 512 tokens, batch 1 / 2 / 4 (128 / 256 / 512 wide workgroups): forward
+// 17.0 -> 14.2, 19.5 -> 17.9, 27.5 -> 31.7 us; dQ + dK/dV passes with the narrow dQ 38.8 -> 37.9, 59.4 -> 54.1,
+// 86.4 -> 90.3 us.  The dK / dV pass needs more than 256 registers either way (one workgroup per CU) and was
+// measured narrow at batch 1 only (63.7 -> 39.4 us for both passes, together with the dQ pass).
+#ifndef BR_FA_SPLIT_UP_TO
+#define BR_FA_SPLIT_UP_TO 256
 #endif
 #ifndef BR_FA_DKV_SPLIT_BELOW
 #define BR_FA_DKV_SPLIT_BELOW 256
 #endif
-inline bool narrow_split(unsigned workgroups) { return workgroups < (unsigned)BR_FA_SPLIT_BELOW; }
+inline bool narrow_split(unsigned workgroups) { return workgroups <= (unsigned)BR_FA_SPLIT_UP_TO; }
 inline bool narrow_split_dkv(unsigned workgroups) { return workgroups < (unsigned)BR_FA_DKV_SPLIT_BELOW; }
 
 bool flash_shape_ok(int64_t batch, int64_t heads, int64_t tokens, int64_t head_dim, int64_t row, int64_t head,
