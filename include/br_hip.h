@@ -374,8 +374,9 @@ int br_hip_linear_residual(const void* x, int x_dtype, const void* w, int w_dtyp
  * alibi: fp32 [heads, tokens] (br_hip_alibi_table); valid: device int32 [batch].
  * lse[batch, heads, tokens] receives log sum exp of each score row, which the
  * backward needs.  Probabilities are rounded to `dtype` before the product
- * with v.  BR_ERR_TODO unless head_dim == 128, strides % 8 == 0
- * and 16-byte aligned bases: callers then run the unfused chain. */
+ * with v.  BR_ERR_TODO unless head_dim == 128, strides % 8 == 0, token
+ * strides below 2^24 elements and 16-byte aligned bases: callers then run
+ * the unfused chain. */
 int br_hip_flash_attn_fwd(const void* q, const void* k, const void* v, int dtype, const float* alibi,
                           const int32_t* valid, void* o, float* lse, int64_t batch, int64_t heads,
                           int64_t tokens, int64_t head_dim, int64_t row_stride, int64_t head_stride,
