@@ -870,6 +870,55 @@ ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& s
     return din->op_add(din, residual, din);
 }
 
+// `op.layernorm_backward_add` followed by the `op.linear_backward` whose dy is the LayerNorm's din: the
+// LayerNorm kernel has every row of din in registers, so it also writes the 16-bit image the two products read
+// and the partial column sums that make the bias gradient -- the pass over din that op.linear_backward starts
+// with does not run.  Anything the fused kernel declines runs as the two operators.
+ComputingReturn hip_layernorm_backward_add_linear_backward(
+    const tensor_t& dy, const tensor_t& scale, const tensor_t& bias, const tensor_t& var, const tensor_t& y,
+    const tensor_t& dscale, const tensor_t& dbias, const tensor_t& residual, const tensor_t& din, float eps,
+    const tensor_t& x, const tensor_t& weight, const tensor_t& lbias, const tensor_t& x_g, const tensor_t& weight_g,
+    const tensor_t& bias_g) {
+    bool fast = dev_f32(dy) && dev_f32(scale) && dev_f32(bias) && dev_f32(var) && dev_f32(y) && dev_f32(dscale) &&
+                dev_f32(dbias) && dev_f32(residual) && dev_f32(din) && dy->shape().dim() == 3 && dev(x) &&
+                dev(weight) && dev(x_g) && dev(weight_g) && dev_f32(bias_g) && x->shape().dim() == 3 &&
+                din->shape().dim() == 3;
+    if (fast) {
+        const int64_t rows = (int64_t)(dy->shape()[0] * dy->shape()[1]);
+        const int64_t cols = (int64_t)dy->shape()[2], in = (int64_t)x->shape()[2];
+        const int compute = pick_compute({din, x, weight});
+        fast = y->items() == dy->items() && (int64_t)var->items() >= rows && din->items() == dy->items() &&
+               residual->items() == dy->items() && (int64_t)dscale->items() == cols && (int64_t)dbias->items() == cols &&
+               (int64_t)scale->items() == cols && (int64_t)bias->items() == cols && din->data() != y->data() &&
+               compute != BR_GEMM_F32 && cols % 8 == 0 && (int64_t)x->items() == rows * in &&
+               (int64_t)weight->items() == cols * in && (int64_t)x_g->items() == rows * in &&
+               (int64_t)weight_g->items() == cols * in && (int64_t)bias_g->items() == cols &&
+               // the gradients this call writes must not be each other or an input of the products
+               bias_g->data() != dscale->data() && bias_g->data() != dbias->data();
+        if (fast) {
+            const int native = compute == BR_GEMM_F16 ? BR_F16 : BR_BF16;
+            const size_t need = br_hip_layernorm_bwd_sums_workspace(rows, cols);
+            void* ws = need <= head_bytes() ? ComputingContext::workspace : ComputingContext::scratch(need);
+            void* d16 = ComputingContext::gemm_staging(1, (size_t)(rows * cols) * 2);
+            const int rc = br_hip_layernorm_bwd_residual_sums(
+                static_cast<const float*>(dy->data()), static_cast<const float*>(y->data()),
+                static_cast<const float*>(scale->data()), static_cast<const float*>(bias->data()),
+                static_cast<const float*>(var->data()), static_cast<const float*>(residual->data()),
+                static_cast<float*>(dscale->data()), static_cast<float*>(dbias->data()),
+                static_cast<float*>(din->data()), d16, native, static_cast<float*>(bias_g->data()), rows, cols, eps,
+                unlift(), ws, need, stream());
+            if (rc != BR_ERR_TODO) {
+                BR_OP(rc);
+                BR_OP(linear_backward_products(Operand{d16, native}, x, weight, x_g, weight_g, rows, in, cols, compute));
+                return OP_OK;
+            }
+        }
+    }
+    const ComputingReturn r = hip_layernorm_backward_add(dy, scale, bias, var, y, dscale, dbias, residual, din, eps);
+    if (r != OP_OK) return r;
+    return din->op_linear_backward(din, x, weight, lbias, x_g, weight_g, bias_g);
+}
+
 template struct HIPTensor<DataType::Float>;
 template struct HIPTensor<DataType::F16>;
 template struct HIPTensor<DataType::BF16>;

@@ -94,5 +94,12 @@ ComputingReturn hip_layernorm_backward_add(const tensor_t& dy, const tensor_t& s
                                            const tensor_t& var, const tensor_t& y, const tensor_t& dscale,
                                            const tensor_t& dbias, const tensor_t& residual, const tensor_t& din,
                                            float eps);
+// The same followed by the linear backward whose output gradient is din (x, weight, bias of that layer and its
+// three gradients): din's 16-bit image and the bias gradient come out of the LayerNorm kernel.
+ComputingReturn hip_layernorm_backward_add_linear_backward(
+    const tensor_t& dy, const tensor_t& scale, const tensor_t& bias, const tensor_t& var, const tensor_t& y,
+    const tensor_t& dscale, const tensor_t& dbias, const tensor_t& residual, const tensor_t& din, float eps,
+    const tensor_t& x, const tensor_t& weight, const tensor_t& lbias, const tensor_t& x_g, const tensor_t& weight_g,
+    const tensor_t& bias_g);
 
 }  // namespace br

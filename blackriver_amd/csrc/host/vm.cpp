@@ -358,6 +358,9 @@ void Enviroment::fuse(DaG& dag) {
                 const DaG::Step& s = dag.steps_[pc];
                 if (s.kind == DaG::Step::RunNative && s.str == seq[at.size()]) {
                     at.push_back(pc);
+                } else if (s.kind == DaG::Step::PushNumber && pc + 1 < dag.steps_.size() &&
+                           dag.steps_[pc + 1].kind == DaG::Step::RunBuiltin && dag.steps_[pc + 1].str == "#") {
+                    pc++;   // `n #`: a switch of the name scope
                 } else if (!is_push(s)) {
                     break;
                 }

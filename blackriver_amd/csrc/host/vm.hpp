@@ -217,7 +217,9 @@ struct Enviroment {
     void insert_native_word(const std::string& name, NativeCreator* fn);
     // Registers a fusion: wherever a linked program runs the native words
     // `sequence` one after the other with nothing but operand pushes
-    // (strings and `@`) in between, the earlier words are skipped -- their
+    // (strings and `@`) and switches of the name scope (`n #`, which
+    // neither touch a tensor nor leave anything on the stack: operands
+    // already pushed are tensors, not names) in between, the earlier words are skipped -- their
     // operands simply stay on the stack -- and the last one is replaced by
     // `fused`, which pops the operands of the whole sequence (first word's
     // deepest) and must produce exactly what the sequence would have.

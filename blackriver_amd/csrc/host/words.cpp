@@ -408,6 +408,22 @@ BR_WORD(LayernormBackwardAdd,
     op_check_word(hip_layernorm_backward_add(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], a[8], eps),
                   "op.layernorm_backward_add");
 )
+// ( dy scale bias var y dscale dbias residual din eps   din' x w b x_g w_g b_g -- )  `op.layernorm_backward_add`
+// followed by the `op.linear_backward` of the layer below; fused when din' is din
+BR_WORD(LayernormBackwardAddLinearBackward,
+    Tensors<7> l(stack);
+    const float eps = (float)stack.pop_number();
+    Tensors<9> a(stack);
+    if (l[0]->data() == a[8]->data() && l[0]->items() == a[8]->items()) {
+        op_check_word(hip_layernorm_backward_add_linear_backward(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], a[8], eps,
+                                                                 l[1], l[2], l[3], l[4], l[5], l[6]),
+                      "op.layernorm_backward_add + op.linear_backward");
+    } else {
+        op_check_word(hip_layernorm_backward_add(a[0], a[1], a[2], a[3], a[4], a[5], a[6], a[7], a[8], eps),
+                      "op.layernorm_backward_add");
+        l[0]->op_linear_backward(l[0], l[1], l[2], l[3], l[4], l[5], l[6]);
+    }
+)
 
 // AdamW on one parameter tensor.  The reference stops at the gradients; these
 // two words are what a training loop runs after them.
@@ -500,6 +516,7 @@ void load_nn_words(Enviroment& env) {
         {"op.linear_gelu", LinearGelu::creator},
         {"op.linear_residual", LinearResidual::creator},
         {"op.layernorm_backward_add", LayernormBackwardAdd::creator},
+        {"op.layernorm_backward_add_linear_backward", LayernormBackwardAddLinearBackward::creator},
         {"op.flash_attn", FlashAttn::creator},
         {"op.flash_attn_backward", FlashAttnBackward::creator},
         {"op.flash_attn_qkv", FlashAttnQkv::creator},
@@ -513,6 +530,7 @@ void load_nn_words(Enviroment& env) {
     env.insert_fusion({"op.add", "op.add", "op.softmax"}, "op.add_add_softmax");
     env.insert_fusion({"op.layernorm", "op.copy"}, "op.layernorm_copy");
     env.insert_fusion({"op.gelu_backward", "op.linear_backward"}, "op.gelu_linear_backward");
+    env.insert_fusion({"op.layernorm_backward_add", "op.linear_backward"}, "op.layernorm_backward_add_linear_backward");
 }
 
 }  // namespace br

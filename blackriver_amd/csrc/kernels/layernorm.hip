@@ -118,8 +118,11 @@ __global__ __launch_bounds__(kBlock) void ln_fwd_generic(const float* x, const f
 // loads in flight while it works on the current one.  At the end the walkers'
 // running sums are added in LDS (walker order) and the workgroup writes ONE
 // partial row pair, so the finalize pass reads gridDim.x partials.
+// SUMS: the finished input gradient (residual included) is also summed over the rows, column by column, into a
+// third partial row, and written a second time in 16 bit: what the backward of the linear layer that produced the
+// LayerNorm's input needs of it (its bias gradient and the operand of its two products).
 constexpr int kWalker = kBlock;  // threads per row walker
-template <int VPT, int GROUPS>
+template <int VPT, int GROUPS, bool SUMS = false>
 __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy, const float* __restrict__ y,
                                                                  const float* __restrict__ gamma,
                                                                  const float* __restrict__ beta,
@@ -127,11 +130,17 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
                                                                  float* __restrict__ part_dgamma,
                                                                  float* __restrict__ part_dbeta, int64_t rows,
                                                                  int cols4, float eps, float inv_cols,
-                                                                 const float* residual) {
+                                                                 const float* residual,
+                                                                 float* __restrict__ part_dx = nullptr,
+                                                                 Copy16 dx16 = Copy16{nullptr, 0}) {
     __shared__ float lds[2][GROUPS][2 * kWaves];
     const int walker = threadIdx.x / kWalker, tid = threadIdx.x % kWalker;
     const int lane = tid & 63, wave = tid >> 6;
-    float4 g[VPT], ginv[VPT], b[VPT], acc_g[VPT], acc_b[VPT];
+    float4 g[VPT], ginv[VPT], b[VPT], acc_g[VPT], acc_b[VPT], acc_x[SUMS ? VPT : 1];
+    if (SUMS) {
+#pragma unroll
+        for (int i = 0; i < VPT; i++) acc_x[SUMS ? i : 0] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int idx = tid + i * kWalker;
@@ -229,6 +238,11 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
                     o.x += res[i].x; o.y += res[i].y; o.z += res[i].z; o.w += res[i].w;
                 }
                 dxr[idx] = o;  // an ordinary store: measured faster here than the streaming form
+                if (SUMS) {
+                    store4_as16(dx16, row * cols4 + idx, o);   // o as stored, rounded once more
+                    float4& ax = acc_x[SUMS ? i : 0];
+                    ax.x += o.x; ax.y += o.y; ax.z += o.z; ax.w += o.w;
+                }
             }
         }
 #pragma unroll
@@ -239,7 +253,7 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
     }
     // walkers 1.. hand their running sums to walker 0 through LDS, in walker order
     if (GROUPS > 1) {
-        __shared__ float4 hand[2][VPT][kWalker];
+        __shared__ float4 hand[SUMS ? 3 : 2][VPT][kWalker];
         for (int w = 1; w < GROUPS; w++) {
             __syncthreads();
             if (walker == w) {
@@ -247,6 +261,7 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
                 for (int i = 0; i < VPT; i++) {
                     hand[0][i][tid] = acc_g[i];
                     hand[1][i][tid] = acc_b[i];
+                    if (SUMS) hand[SUMS ? 2 : 0][i][tid] = acc_x[SUMS ? i : 0];
                 }
             }
             __syncthreads();
@@ -256,6 +271,11 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
                     const float4 a = hand[0][i][tid], c = hand[1][i][tid];
                     acc_g[i].x += a.x; acc_g[i].y += a.y; acc_g[i].z += a.z; acc_g[i].w += a.w;
                     acc_b[i].x += c.x; acc_b[i].y += c.y; acc_b[i].z += c.z; acc_b[i].w += c.w;
+                    if (SUMS) {
+                        const float4 e = hand[SUMS ? 2 : 0][i][tid];
+                        float4& ax = acc_x[SUMS ? i : 0];
+                        ax.x += e.x; ax.y += e.y; ax.z += e.z; ax.w += e.w;
+                    }
                 }
             }
         }
@@ -269,6 +289,7 @@ __global__ __launch_bounds__(kWalker * GROUPS) void ln_bwd_regs(const float* dy,
             if (idx < cols4) {
                 pg[idx] = acc_g[i];
                 pb[idx] = acc_b[i];
+                if (SUMS) reinterpret_cast<float4*>(part_dx)[(int64_t)blockIdx.x * cols4 + idx] = acc_x[SUMS ? i : 0];
             }
         }
     }
@@ -346,43 +367,41 @@ __global__ __launch_bounds__(kBlock) void ln_bwd_finalize(const float* part_dgam
 // all of a workgroup's loads are in flight at once; slices are combined in LDS
 // in a fixed order.
 constexpr int kFinSlices = 64;
-__global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restrict__ part_dgamma,
-                                                           const float4* __restrict__ part_dbeta,
-                                                           float4* __restrict__ dgamma, float4* __restrict__ dbeta,
+struct FinalSums {
+    float4* out[3];   // dgamma, dbeta and (or null) the column sums of dx
+};
+// blockIdx.y picks the array: the partial arrays lie one after the other, parts x cols4 quads each
+__global__ __launch_bounds__(1024) void ln_bwd_finalize_x4(const float4* __restrict__ partials, FinalSums sums,
                                                            int parts, int cols4, float scale) {
-    __shared__ float4 lg[kFinSlices][16], lb[kFinSlices][16];
+    __shared__ float4 ls[kFinSlices][16];
+    const float4* __restrict__ part = partials + (int64_t)blockIdx.y * parts * cols4;
+    float4* __restrict__ out = sums.out[blockIdx.y];
     const int q = threadIdx.x & 15, sl = threadIdx.x >> 4;
     const int c4 = blockIdx.x * 16 + q;
-    float4 sg = make_float4(0.f, 0.f, 0.f, 0.f), sb = sg;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
     if (c4 < cols4) {
 #pragma unroll 8
         for (int p = sl; p < parts; p += kFinSlices) {
-            const float4 a = part_dgamma[(int64_t)p * cols4 + c4], b = part_dbeta[(int64_t)p * cols4 + c4];
-            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
-            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+            const float4 a = part[(int64_t)p * cols4 + c4];
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
         }
     }
-    lg[sl][q] = sg;
-    lb[sl][q] = sb;
+    ls[sl][q] = s;
     __syncthreads();
     if (sl < 8) {
         for (int k = sl + 8; k < kFinSlices; k += 8) {
-            const float4 a = lg[k][q], b = lb[k][q];
-            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
-            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+            const float4 a = ls[k][q];
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
         }
-        lg[sl][q] = sg;
-        lb[sl][q] = sb;
+        ls[sl][q] = s;
     }
     __syncthreads();
     if (sl == 0 && c4 < cols4) {
         for (int k = 1; k < 8; k++) {
-            const float4 a = lg[k][q], b = lb[k][q];
-            sg.x += a.x; sg.y += a.y; sg.z += a.z; sg.w += a.w;
-            sb.x += b.x; sb.y += b.y; sb.z += b.z; sb.w += b.w;
+            const float4 a = ls[k][q];
+            s.x += a.x; s.y += a.y; s.z += a.z; s.w += a.w;
         }
-        dgamma[c4] = make_float4(sg.x * scale, sg.y * scale, sg.z * scale, sg.w * scale);
-        dbeta[c4] = make_float4(sb.x * scale, sb.y * scale, sb.z * scale, sb.w * scale);
+        out[c4] = make_float4(s.x * scale, s.y * scale, s.z * scale, s.w * scale);
     }
 }
 
@@ -497,49 +516,74 @@ size_t br_hip_layernorm_bwd_workspace(int64_t rows, int64_t cols) {
     return (size_t)(2 * parts * cols) * sizeof(float);
 }
 
+size_t br_hip_layernorm_bwd_sums_workspace(int64_t rows, int64_t cols) {
+    return br_hip_layernorm_bwd_workspace(rows, cols) / 2 * 3;   // a third partial array
+}
+
+// dx16 / dx_sum (both or neither): the 16-bit copy and the column sums of dx, register path only
 static int layernorm_bwd_impl(const float* dy, const float* y, const float* gamma, const float* beta,
                               const float* var, const float* residual, float* dgamma, float* dbeta, float* dx,
                               int64_t rows, int64_t cols, float eps, float param_scale, void* workspace,
-                              size_t workspace_bytes, br_stream_t stream) {
+                              size_t workspace_bytes, br_stream_t stream, void* dx16 = nullptr, int dx16_dtype = 0,
+                              float* dx_sum = nullptr) {
     if (rows < 0 || cols <= 0 || rows > 0x7fffffff) return BR_ERR_ATTR;
     if (!dgamma || !dbeta) return BR_ERR_OUTPUT;
+    const bool sums = dx_sum != nullptr;
     if (rows == 0) {
         int rc = br_hip_fill(dgamma, BR_F32, 0.f, cols, stream);
+        if (!rc && sums) rc = br_hip_fill(dx_sum, BR_F32, 0.f, cols, stream);
         return rc ? rc : br_hip_fill(dbeta, BR_F32, 0.f, cols, stream);
     }
     if (!dy || !y || !gamma || !beta || !var) return BR_ERR_INPUT;
     if (!dx) return BR_ERR_OUTPUT;
-    if (!workspace || workspace_bytes < br_hip_layernorm_bwd_workspace(rows, cols)) return BR_ERR_ATTR;
+    const size_t need = sums ? br_hip_layernorm_bwd_sums_workspace(rows, cols) : br_hip_layernorm_bwd_workspace(rows, cols);
+    if (!workspace || workspace_bytes < need) return BR_ERR_ATTR;
     hipStream_t st = as_stream(stream);
     int parts;
     float* part_g = (float*)workspace;
     const bool regs = regs_path_ok(cols, dy, y, gamma, beta, dx) && aligned16(workspace) &&
                       (!residual || aligned16(residual));
     if (residual && !regs) return BR_ERR_TODO;  // only the register path adds the residual
+    const int cols4 = (int)(cols / 4);
+    const int vpt = (cols4 + kBlock - 1) / kBlock;
+    // ... and the sums: up to 4096 columns (wider rows run one walker with every register taken), all of dgamma,
+    // dbeta and the sums aligned for the finalize pass that handles three arrays
+    if (sums && !(regs && vpt <= 4 && aligned16(dgamma) && aligned16(dbeta) && aligned16(dx_sum) &&
+                  copy16_ok(dx16, dx16_dtype)))
+        return BR_ERR_TODO;
     if (regs) {
         parts = bwd_parts(rows);
         float* part_b = part_g + (int64_t)parts * cols;
-        const int cols4 = (int)(cols / 4);
+        float* part_x = part_b + (int64_t)parts * cols;
         const float inv = 1.0f / (float)cols;
-        const int vpt = (cols4 + kBlock - 1) / kBlock;
         constexpr int G = kBwdWalkers;
-#define BR_LN_BWD(V, W)                                                                                           \
-    ln_bwd_regs<V, W><<<parts, kWalker * W, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps, \
-                                                     inv, residual)
+        const Copy16 c16{dx16, dx16_dtype == BR_BF16};
+#define BR_LN_BWD(V, W)                                                                                              \
+    do {                                                                                                             \
+        if (sums)                                                                                                    \
+            ln_bwd_regs<V, W, true><<<parts, kWalker * W, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, \
+                                                                   cols4, eps, inv, residual, part_x, c16);          \
+        else                                                                                                         \
+            ln_bwd_regs<V, W><<<parts, kWalker * W, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows,      \
+                                                             cols4, eps, inv, residual);                             \
+    } while (0)
         // Rows wider than 4096 floats keep 8 quads per thread in flight twice over; with two walkers (512
         // threads, 256 registers per wave) that spills, so they run one walker per workgroup.
         if (vpt <= 1) BR_LN_BWD(1, G);
         else if (vpt <= 2) BR_LN_BWD(2, G);
         else if (vpt <= 4) BR_LN_BWD(4, G);
-        else BR_LN_BWD(8, 1);
+        else ln_bwd_regs<8, 1><<<parts, kWalker, 0, st>>>(dy, y, gamma, beta, var, dx, part_g, part_b, rows, cols4, eps,
+                                                          inv, residual);
 #undef BR_LN_BWD
         BR_HIP_LAUNCH_CHECK();
-        if (aligned16(dgamma) && aligned16(dbeta))
-            ln_bwd_finalize_x4<<<(unsigned)((cols4 + 15) / 16), 1024, 0, st>>>(
-                reinterpret_cast<const float4*>(part_g), reinterpret_cast<const float4*>(part_b),
-                reinterpret_cast<float4*>(dgamma), reinterpret_cast<float4*>(dbeta), parts, cols4, param_scale);
-        else
+        if (aligned16(dgamma) && aligned16(dbeta)) {
+            const FinalSums out{{reinterpret_cast<float4*>(dgamma), reinterpret_cast<float4*>(dbeta),
+                                 reinterpret_cast<float4*>(dx_sum)}};
+            ln_bwd_finalize_x4<<<dim3((unsigned)((cols4 + 15) / 16), sums ? 3u : 2u), 1024, 0, st>>>(
+                reinterpret_cast<const float4*>(part_g), out, parts, cols4, param_scale);
+        } else {
             ln_bwd_finalize<<<(unsigned)((cols + 63) / 64), kBlock, 0, st>>>(part_g, part_b, dgamma, dbeta, parts, cols, param_scale);
+        }
     } else {
         const int rpb = strip_rows(rows);
         parts = (int)((rows + rpb - 1) / rpb);
@@ -579,6 +623,18 @@ int br_hip_layernorm_bwd_static(const float* dy, const float* y, const float* ga
     // same call, so nothing in the array has to start at zero
     return layernorm_bwd_impl(dy, y, gamma, beta, var, nullptr, dgamma, dbeta, dx, rows, cols, eps, param_scale, ws,
                               kStaticScratchBytes, stream);
+}
+
+int br_hip_layernorm_bwd_residual_sums(const float* dy, const float* y, const float* gamma, const float* beta,
+                                       const float* var, const float* residual, float* dgamma, float* dbeta,
+                                       float* dx, void* dx16, int dx16_dtype, float* dx_sum, int64_t rows,
+                                       int64_t cols, float eps, float param_scale, void* workspace,
+                                       size_t workspace_bytes, br_stream_t stream) {
+    if (rows > 0 && !residual) return BR_ERR_INPUT;
+    if (!dx16 || !dx_sum) return BR_ERR_OUTPUT;
+    if (rows == 0) residual = nullptr;
+    return layernorm_bwd_impl(dy, y, gamma, beta, var, residual, dgamma, dbeta, dx, rows, cols, eps, param_scale,
+                              workspace, workspace_bytes, stream, dx16, dx16_dtype, dx_sum);
 }
 
 int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* gamma, const float* beta,

@@ -67,6 +67,8 @@ SIGNATURES = {
     "br_hip_layernorm_bwd_static": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _f32, _f32, _vp]),
     "br_hip_layernorm_bwd_static_limit": (_sz, []),
     "br_hip_layernorm_bwd_residual": (_int, [_vp] * 9 + [_i64, _i64, _f32, _f32, _vp, _sz, _vp]),
+    "br_hip_layernorm_bwd_sums_workspace": (_sz, [_i64, _i64]),
+    "br_hip_layernorm_bwd_residual_sums": (_int, [_vp] * 10 + [_int, _vp, _i64, _i64, _f32, _f32, _vp, _sz, _vp]),
     "br_hip_softmax_fwd": (_int, [_vp, _vp, _i64, _i64, _vp]),
     "br_hip_softmax_bwd": (_int, [_vp, _vp, _vp, _i64, _i64, _vp]),
     "br_hip_softmax_bwd_to16": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _vp]),

@@ -213,6 +213,24 @@ int br_hip_layernorm_bwd_residual(const float* dy, const float* y, const float* 
                                   int64_t cols, float eps, float param_scale, void* workspace,
                                   size_t workspace_bytes, br_stream_t stream);
 
+/* The same followed by what the `op.linear_backward` of the layer below does to
+ * dx first (cuda_tensor.cpp:738-760: its bias gradient, the column sums of dx;
+ * and, for 16-bit products, the 16-bit image of dx both of its products read):
+ * dx16 = dx rounded to dx16_dtype (BR_F16 / BR_BF16), dx_sum[c] = param_scale *
+ * sum over rows of dx[r, c], the sums in a fixed order.  dx16 and dx are what
+ * br_hip_colsum_cast would make of dx; the sums agree with its to rounding (a
+ * different but equally fixed summation order).  Workspace:
+ * br_hip_layernorm_bwd_sums_workspace.  BR_ERR_TODO for rows wider than 4096
+ * columns, unaligned dgamma / dbeta / dx_sum / dx16 and whatever
+ * br_hip_layernorm_bwd_residual declines: callers then run the two steps. */
+size_t br_hip_layernorm_bwd_sums_workspace(int64_t rows, int64_t cols);
+int br_hip_layernorm_bwd_residual_sums(const float* dy, const float* y, const float* gamma,
+                                       const float* beta, const float* var, const float* residual,
+                                       float* dgamma, float* dbeta, float* dx, void* dx16,
+                                       int dx16_dtype, float* dx_sum, int64_t rows, int64_t cols,
+                                       float eps, float param_scale, void* workspace,
+                                       size_t workspace_bytes, br_stream_t stream);
+
 /* ---- softmax family ---------------------------------------------------- */
 /* cudnnSoftmaxForward(ACCURATE, INSTANCE) at cuda_tensor.cpp:332-356 and
  * cudnnSoftmaxBackward at :890-918.  y may alias x; dx may alias dy. */

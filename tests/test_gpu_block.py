@@ -523,6 +523,75 @@ def test_fused_gelu_backward_linear_backward_equals_the_two_words(runtime, mode)
         env.close()
 
 
+@pytest.mark.parametrize("mode,hidden", [("f16", 256), ("bf16", 256), ("f32", 256), ("f16", 8192)])
+def test_fused_layernorm_backward_add_linear_backward_equals_the_two_words(runtime, mode, hidden):
+    """The fusion pass turns `op.layernorm_backward_add op.linear_backward` (the post-attention LayerNorm's
+    backward followed by the dense layer's in the block's backward) into one word when the second reads the
+    gradient the first writes.  Fused (one program) and unfused (two programs) must agree: the LayerNorm's
+    outputs, the 16-bit products' results (they read the same 16-bit image) bit for bit, the bias gradient to
+    the rounding of a different summation order; in fp32 mode and on rows wider than the fused kernel takes the
+    word falls back to the two operators (same bits throughout); a pair that is not chained is left alone."""
+    rng = np.random.default_rng(23)
+    b, t, inner = 2, 24, 128
+    env = host.Env(1)
+    try:
+        env.execute("'%s' op.gemm_precision" % mode)
+        wdt = {"f16": "f16", "bf16": "bf16", "f32": "float"}[mode]
+        for n in ("dy", "ln", "res", "din", "other"):
+            env.execute("%d %d %d 3 'cuda' 'float' op.create '%s' !" % (b, t, hidden, n))
+        env.execute("%d %d %d 3 'cuda' '%s' op.create 'x' !  %d %d %d 3 'cuda' 'float' op.create 'xg' !"
+                    % (b, t, inner, wdt, b, t, inner))
+        env.execute("%d %d 2 'cuda' '%s' op.create 'w' !  %d %d 2 'cuda' 'float' op.create 'wg' !"
+                    % (hidden, inner, wdt, hidden, inner))
+        for n in ("gam", "bet", "dgam", "dbet", "bias", "bg"):
+            env.execute("%d 1 'cuda' 'float' op.create '%s' !" % (hidden, n))
+        env.execute("%d 1 'cuda' 'float' op.create 'var' !  %d 1 'cuda' 'float' op.create 'mean' !" % (b * t, b * t))
+        env.write("gam", (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32))
+        env.write("bet", (0.1 * rng.standard_normal(hidden)).astype(np.float32))
+        env.write("other", rng.standard_normal((b, t, hidden)).astype(np.float32))
+        env.execute("'other' @ 'mean' @ 'var' @ 'gam' @ 'bet' @ 'ln' @ 1e-5 op.layernorm")
+        env.write("dy", rng.standard_normal((b, t, hidden)).astype(np.float32))
+        env.write("res", rng.standard_normal((b, t, hidden)).astype(np.float32))
+        env.write("x", rng.standard_normal((b, t, inner)).astype(np.float32))
+        env.write("w", (0.05 * rng.standard_normal((hidden, inner))).astype(np.float32))
+        ln = "'dy' @ 'gam' @ 'bet' @ 'var' @ 'ln' @ 'dgam' @ 'dbet' @ 'res' @ 'din' @ 1e-5 op.layernorm_backward_add"
+        lin = "'din' @ 'x' @ 'w' @ 'bias' @ 'xg' @ 'wg' @ 'bg' @ op.linear_backward"
+        assert "W:op.layernorm_backward_add_linear_backward" in env.disassemble(ln + "  " + lin, fused=True)
+        # a switch of the name scope between the two (the model driver goes from one block's words to the next
+        # block's that way) does not hide the pair; anything else does
+        assert "W:op.layernorm_backward_add_linear_backward" in env.disassemble(ln + "  0 #  " + lin, fused=True)
+        assert "W:op.layernorm_backward_add_linear_backward" not in env.disassemble(ln + "  op.sync  " + lin, fused=True)
+        assert "W:op.layernorm_backward_add_linear_backward" not in env.disassemble(ln + "  7  " + lin, fused=True)
+        outs = ("din", "dgam", "dbet", "xg", "wg", "bg")
+        zero = "  ".join("'%s' @ op.zero" % n for n in outs)
+        env.execute(zero)
+        env.execute(ln)
+        env.execute(lin)
+        want = {n: env.read(n) for n in outs}
+        env.execute(zero)
+        env.execute(ln + "  0 #  " + lin)
+        for n in outs:
+            got = env.read(n)
+            if n == "bg" and mode != "f32" and hidden <= 4096:
+                # the fused kernel's column sums: another fixed order
+                mag = np.abs(want["din"]).reshape(-1, hidden).sum(0)
+                assert np.all(np.abs(got - want[n]) <= 2e-6 * mag + 1e-30), (mode, n)
+            else:
+                assert np.array_equal(got, want[n]), (mode, hidden, n)
+        # the linear backward of some other gradient: the word must run the pair as written
+        lin2 = "'other' @ 'x' @ 'w' @ 'bias' @ 'xg' @ 'wg' @ 'bg' @ op.linear_backward"
+        env.execute(zero)
+        env.execute(ln)
+        env.execute(lin2)
+        want = {n: env.read(n) for n in outs}
+        env.execute(zero)
+        env.execute(ln + "  " + lin2)
+        for n in outs:
+            assert np.array_equal(env.read(n), want[n]), (mode, hidden, n, "unchained")
+    finally:
+        env.close()
+
+
 def test_fused_attention_follows_the_mask_tables_prefix_rule(runtime):
     """A mask with a hole: the reference's table closes every key from the
     first zero on (train_bloom.cpp:73-90), so `bloom.valid` must report the

@@ -167,6 +167,52 @@ def test_layernorm_bwd_with_residual_equals_backward_then_add(rows, cols):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("dtype,tdtype", [(F16, torch.float16), (BF16, torch.bfloat16)])
+@pytest.mark.parametrize("rows,cols", [(2048, 4096), (512, 4096), (37, 1024), (3, 256)])
+def test_layernorm_bwd_with_residual_sums_and_16_bit_copy(rows, cols, dtype, tdtype):
+    """The backward + residual that also leaves the 16-bit image and the column sums of its result (the first pass
+    of the linear backward below it): dx, dgamma, dbeta bit for bit those of br_hip_layernorm_bwd_residual, the
+    image bit for bit dx rounded once, the sums (times param_scale) against a float64 sum of dx as stored --
+    through the lifted-gradient factor too."""
+    print("case rows=%d cols=%d dtype=%d" % (rows, cols, dtype), flush=True)
+    x, g, b, dy = make(rows, cols, seed=7)
+    res = np.random.default_rng(8).standard_normal((rows, cols)).astype(np.float32)
+    eps = 1e-5
+    y_ref, _, var_ref = orc.layernorm_fwd(x, g, b, eps)
+    lib = hip.load()
+    ws = workspace(lib.br_hip_layernorm_bwd_sums_workspace(rows, cols))
+    assert lib.br_hip_layernorm_bwd_sums_workspace(rows, cols) >= lib.br_hip_layernorm_bwd_workspace(rows, cols)
+    for scale in (1.0, 1.0 / 1024):
+        t_dy, t_y, t_g, t_b, t_var, t_res = (dev(a) for a in (dy, y_ref, g, b, var_ref, res))
+        dgam, dbet, dx = empty(cols), empty(cols), empty((rows, cols))
+        call("br_hip_layernorm_bwd_residual", ptr(t_dy), ptr(t_y), ptr(t_g), ptr(t_b), ptr(t_var), ptr(t_res),
+             ptr(dgam), ptr(dbet), ptr(dx), rows, cols, eps, scale, ptr(ws), ws.numel(), stream())
+        dgam2, dbet2, dx2, sums = empty(cols), empty(cols), empty((rows, cols)), empty(cols)
+        dx16 = torch.zeros((rows, cols), dtype=tdtype, device="cuda")
+        call("br_hip_layernorm_bwd_residual_sums", ptr(t_dy), ptr(t_y), ptr(t_g), ptr(t_b), ptr(t_var), ptr(t_res),
+             ptr(dgam2), ptr(dbet2), ptr(dx2), ptr(dx16), dtype, ptr(sums), rows, cols, eps, scale, ptr(ws), ws.numel(),
+             stream())
+        assert torch.equal(dx2, dx) and torch.equal(dgam2, dgam) and torch.equal(dbet2, dbet)
+        assert torch.equal(dx16, dx.to(tdtype))
+        want = host(dx).astype(np.float64).sum(0) * scale
+        # fp32 sums in a fixed tree: a few ulps of the sum of magnitudes
+        bound = 1e-6 * np.abs(host(dx)).astype(np.float64).sum(0) * scale + 1e-30
+        assert np.all(np.abs(host(sums) - want) <= bound), float((np.abs(host(sums) - want) / bound).max())
+    # declined: rows wider than 4096 columns, a misaligned sums pointer; missing outputs are an error
+    t = empty(2 * 8192)
+    gg = empty(8192 + 4)
+    h = torch.zeros(2 * 8192, dtype=tdtype, device="cuda")
+    ws2 = workspace(lib.br_hip_layernorm_bwd_sums_workspace(2, 8192))
+    args = lambda sums_ptr, h_ptr, c: (ptr(t), ptr(t), ptr(gg), ptr(gg), ptr(gg), ptr(t), ptr(gg), ptr(gg), ptr(t), h_ptr,
+                                       dtype, sums_ptr, 2, c, eps, 1.0, ptr(ws2), ws2.numel(), stream())
+    assert lib.br_hip_layernorm_bwd_residual_sums(*args(ptr(gg), ptr(h), 8192)) == -1
+    import ctypes
+    assert lib.br_hip_layernorm_bwd_residual_sums(*args(ctypes.c_void_p(gg.data_ptr() + 4), ptr(h), 4096)) == -1
+    assert lib.br_hip_layernorm_bwd_residual_sums(*args(None, ptr(h), 4096)) == -3
+    assert lib.br_hip_layernorm_bwd_residual_sums(*args(ptr(gg), None, 4096)) == -3
+    torch.cuda.synchronize()
+
+
 def test_layernorm_bwd_param_scale_is_an_exact_power_of_two_factor():
     """dy lifted by S = 1024 with param_scale = 1/S: dx comes out S times the
     plain one and dgamma / dbeta equal the plain ones, all bit for bit (scaling
