@@ -795,10 +795,10 @@ __global__ __launch_bounds__(64 * G * KH, 2) void flash_bwd_dq_kernel(FlashArgs 
 
 // Whether a launch that would take `workgroups` workgroups of 128 queries (or keys) runs on twice as many of 64
 // instead, each tile's work split between two waves: where the wider ones would leave compute units empty or with
-// one workgroup each.  Measured at 32 heads x 512 tokens, batch 1 / 2 / 4 (128 / 256 / 512 wide workgroups): forward
-// 17.0 -> 14.2, 19.5 -> 17.9, 27.5 -> 31.7 us; dQ + dK/dV passes with the narrow dQ 38.8 -> 37.9, 59.4 -> 54.1,
-// 86.4 -> 90.3 us.  The dK / dV pass needs more than 256 registers either way (one workgroup per CU) and was
-// measured narrow at batch 1 only (63.7 -> 39.4 us for both passes, together with the dQ pass).
+// one workgroup each.  Measured at 32 heads x 512 tokens, batch 1 / 2 / 4 (128 / 256 / 512 wide workgroups), wide
+// against narrow: forward 19.5 -> 14.2, 19.5 -> 17.9, 27.5 -> 31.7 us; dQ + dK/dV passes 56.0 -> 37.9 (both narrow),
+// 59.4 -> 54.1 and 86.4 -> 90.3 (dQ narrow).  The dK / dV pass needs more than 256 registers either way (one
+// workgroup per CU) and was measured narrow at batch 1 only.
 #ifndef BR_FA_SPLIT_UP_TO
 #define BR_FA_SPLIT_UP_TO 256
 #endif
