@@ -165,11 +165,18 @@ __device__ __forceinline__ void load4_device_coherent(f32x4 (&v)[4], const f32x4
         : "memory");
 }
 
+// KW = 2: the sixteen-wide sub-steps of every K step are dealt to two groups of waves (group kw takes sub-steps
+// kw * KS/2 ..), each group covering the whole tile with wave tiles twice as large; the groups' accumulators are
+// added through LDS after the K loop (group 1 into group 0, which runs the epilogue).  For tiles too small to give
+// eight waves a 64 x 128 block each: a 256 x 128 tile on eight 64 x 64 waves reads 128 KB of fragments per K step
+// from LDS, on two groups of four 64 x 128 waves 96 KB.
 template <int CT, int BM, int BN, int WM, int WN, int KT, int STAGES, bool A_KSTR, bool B_KSTR, typename TC,
-          bool GELU = false, bool SPLIT = false>
-__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(GemmArgs g) {
-    constexpr int WAVES = (BM / WM) * (BN / WN);
-    constexpr int FM = WM / 32, FN = WN / 32, KS = KT / 16;
+          bool GELU = false, bool SPLIT = false, int KW = 1>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * KW * 64) void gemm_dtl_kernel(GemmArgs g) {
+    constexpr int WAVES_MN = (BM / WM) * (BN / WN);
+    constexpr int WAVES = WAVES_MN * KW;
+    constexpr int FM = WM / 32, FN = WN / 32, KS = KT / 16 / KW;   // KS: sub-steps of a K step per wave
+    static_assert(KW == 1 || (KW == 2 && KT == 64 && !SPLIT), "two wave groups: 64-wide K steps, no K split across workgroups");
     using TA = DtlTile<BM, KT, WAVES, A_KSTR>;
     using TB = DtlTile<BN, KT, WAVES, B_KSTR>;
     constexpr int kStageBytes = TA::kBytes + TB::kBytes;
@@ -198,7 +205,8 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
     const long long row0 = (long long)tm * BM, col0 = (long long)tn * BN;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int wm = wave / (BN / WN), wn = wave % (BN / WN);
+    const int kw = KW == 1 ? 0 : wave / WAVES_MN, wave_mn = KW == 1 ? wave : wave % WAVES_MN;
+    const int wm = wave_mn / (BN / WN), wn = wave_mn % (BN / WN);
 
     // tile origins at K step 0 (wave-uniform, advanced once per step) and the
     // per-lane chunk offsets (fixed for the whole K loop)
@@ -218,9 +226,9 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
 #pragma unroll
-        for (int i = 0; i < FM; i++) fa_off[i][ks] = TA::frag_offset(wm * WM + i * 32, ks, lane);
+        for (int i = 0; i < FM; i++) fa_off[i][ks] = TA::frag_offset(wm * WM + i * 32, kw * KS + ks, lane);
 #pragma unroll
-        for (int j = 0; j < FN; j++) fb_off[j][ks] = TA::kBytes + TB::frag_offset(wn * WN + j * 32, ks, lane);
+        for (int j = 0; j < FN; j++) fb_off[j][ks] = TA::kBytes + TB::frag_offset(wn * WN + j * 32, kw * KS + ks, lane);
     }
 
     // this workgroup's K steps: [k_begin, k_begin + nk) of the g.k / KT steps (all of them without a split)
@@ -324,6 +332,37 @@ __global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void gemm_dtl_kernel(Ge
                 step(fa_now, fb_now, fa_next, fb_next, t + 1, 0);
             }
         }
+    }
+
+    if constexpr (KW == 2) {
+        // Every tile issued has landed and been read (the loop's last waits and barrier); the stages now carry
+        // group 1's accumulators to group 0: quad q of thread t of wave w at quad index (w * 4 FM FN + q) * 64 + t.
+        static_assert((size_t)STAGES * kStageBytes >= (size_t)WAVES_MN * FM * FN * 16 * 64 * 4, "the stages hold one group's sums");
+        f32x4* const x = reinterpret_cast<f32x4*>(lds_raw) + (size_t)wave_mn * (4 * FM * FN) * 64 + lane;
+        __syncthreads();   // the last sub-step's (unused) fragment reads are done too
+        if (kw == 1) {
+#pragma unroll
+            for (int i = 0; i < FM; i++)
+#pragma unroll
+                for (int j = 0; j < FN; j++)
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        f32x4 v;
+                        v.x = acc[i][j][4 * q]; v.y = acc[i][j][4 * q + 1]; v.z = acc[i][j][4 * q + 2]; v.w = acc[i][j][4 * q + 3];
+                        x[((i * FN + j) * 4 + q) * 64] = v;
+                    }
+        }
+        __syncthreads();
+        if (kw == 1) return;
+#pragma unroll
+        for (int i = 0; i < FM; i++)
+#pragma unroll
+            for (int j = 0; j < FN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const f32x4 v = x[((i * FN + j) * 4 + q) * 64];
+                    acc[i][j][4 * q] += v.x; acc[i][j][4 * q + 1] += v.y; acc[i][j][4 * q + 2] += v.z; acc[i][j][4 * q + 3] += v.w;
+                }
     }
 
     if constexpr (SPLIT) {
@@ -711,9 +750,15 @@ int launch_dtl_walk(GemmArgs g, const Problem& p, hipStream_t st) {
 }
 
 // ---- host-side dispatch -------------------------------------------------------
-template <int CT, int BM, int BN, int WM, int WN, int KT, int ST>
+#ifndef BR_DTL_KW
+#define BR_DTL_KW 1
+#endif
+#ifndef BR_DTL_KW_MIN_STEPS
+#define BR_DTL_KW_MIN_STEPS 24
+#endif
+template <int CT, int BM, int BN, int WM, int WN, int KT, int ST, int KW = 1>
 int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
-    constexpr int THREADS = (BM / WM) * (BN / WN) * 64;
+    constexpr int THREADS = (BM / WM) * (BN / WN) * KW * 64;
     g.tiles_m = (int)((g.m + BM - 1) / BM);
     g.tiles_n = (int)((g.n + BN - 1) / BN);
     if (g.splits > 1) {
@@ -731,9 +776,9 @@ int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t
     if (g.splits == 2) {
         // the two-slice form: its own instantiations (of the two 256-row tiles, the only ones it is planned on),
         // so that the unsplit kernels carry none of its code
-        if (g.c2 || BM != 256) return BR_ERR_TODO;
+        if (g.c2 || BM != 256 || KW != 1) return BR_ERR_TODO;
 #define BR_DTL_SPLIT_CASE(AK, BK_)                                                                              \
-    if constexpr (BM == 256) if (p.a_kstr == AK && p.b_kstr == BK_) {                                                                     \
+    if constexpr (BM == 256 && KW == 1) if (p.a_kstr == AK && p.b_kstr == BK_) {                                                          \
         if (p.c_dtype == BR_F32)                                                                                 \
             gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, float, false, true><<<grid, THREADS, 0, st>>>(g); \
         else if (CT == BR_GEMM_F16)                                                                              \
@@ -753,20 +798,20 @@ int launch_dtl_config(GemmArgs g, const Problem& p, long long batch, hipStream_t
         // GELU epilogue: built for the linear layer's layout only (both operands k-contiguous, 16-bit outputs)
         if (p.a_kstr || p.b_kstr || p.c_dtype == BR_F32) return BR_ERR_TODO;
         if (CT == BR_GEMM_F16)
-            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, false, false, F16, true><<<grid, THREADS, 0, st>>>(g);
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, false, false, F16, true, false, KW><<<grid, THREADS, 0, st>>>(g);
         else
-            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, false, false, BF16, true><<<grid, THREADS, 0, st>>>(g);
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, false, false, BF16, true, false, KW><<<grid, THREADS, 0, st>>>(g);
         BR_HIP_LAUNCH_CHECK();
         return BR_OK;
     }
 #define BR_DTL_CASE(AK, BK_)                                                                           \
     if (p.a_kstr == AK && p.b_kstr == BK_) {                                                            \
         if (p.c_dtype == BR_F32)                                                                        \
-            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, float><<<grid, THREADS, 0, st>>>(g);   \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, float, false, false, KW><<<grid, THREADS, 0, st>>>(g);   \
         else if (CT == BR_GEMM_F16)                                                                     \
-            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, F16><<<grid, THREADS, 0, st>>>(g);     \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, F16, false, false, KW><<<grid, THREADS, 0, st>>>(g);     \
         else                                                                                            \
-            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, BF16><<<grid, THREADS, 0, st>>>(g);    \
+            gemm_dtl_kernel<CT, BM, BN, WM, WN, KT, ST, AK, BK_, BF16, false, false, KW><<<grid, THREADS, 0, st>>>(g);    \
     }
     BR_DTL_CASE(false, false)
     BR_DTL_CASE(false, true)
@@ -916,12 +961,17 @@ int launch_dtl(GemmArgs g, const Problem& p, long long batch, hipStream_t st) {
         if (g.c2) tail.c2 = static_cast<unsigned char*>(g.c2) + c_size * tail_from;
         if (g.addend) tail.addend = static_cast<const unsigned char*>(g.addend) + c_size * tail_from;
         if (g.bias) tail.bias = g.bias + tail_from;
+        if (BR_DTL_KW && g.k / 64 >= BR_DTL_KW_MIN_STEPS) return launch_dtl_config<CT, 256, 128, 64, 128, 64, 3, 2>(tail, p, batch, st);
         return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(tail, p, batch, st);
     }
     const int pick = plan.config;
     if (pick == 0 && walk_applies(g, batch)) return launch_dtl_walk<CT>(g, p, st);
     if (pick == 0) return launch_dtl_config<CT, 256, 256, 64, 128, 64, 2>(g, p, batch, st);
-    if (pick == 1) return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
+    if (pick == 1) {
+        // long K: two groups of four 64 x 128 waves per tile (fewer fragment reads, a merge at the end)
+        if (BR_DTL_KW && g.k / 64 >= BR_DTL_KW_MIN_STEPS) return launch_dtl_config<CT, 256, 128, 64, 128, 64, 3, 2>(g, p, batch, st);
+        return launch_dtl_config<CT, 256, 128, 64, 64, 64, 3>(g, p, batch, st);
+    }
     if (pick == 2) return launch_dtl_config<CT, 128, 128, 64, 64, 64, 2>(g, p, batch, st);
     return launch_dtl_config<CT, 128, 128, 64, 64, 32, 3>(g, p, batch, st);
 }

@@ -263,6 +263,29 @@ def test_gemm_round_and_a_half_of_tiles(ta, tb, n, c_dt):
 
 
 @pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
+@pytest.mark.parametrize("c_dt", [F32, F16])
+def test_gemm_tile_on_two_groups_of_waves(ta, tb, c_dt):
+    """[1024 x 8192] from K = 2048: 256 tiles of 256 x 128 and 32 K steps, which the dispatcher runs with the
+    sub-steps of every K step dealt to two groups of four waves whose sums meet in LDS after the K loop.  Alpha,
+    bias and an accumulated C; against fp64, and with small-integer operands (every partial sum exact) bit for
+    bit."""
+    rng = np.random.default_rng(33)
+    m, n, k = 1024, 8192, 2048
+    print("case ta=%d tb=%d c_dt=%d" % (ta, tb, c_dt), flush=True)
+    a, b = operands(rng, ta, tb, m, n, k)
+    bias = rng.standard_normal(n).astype(np.float32)
+    c0 = rng.standard_normal((1, m, n)).astype(np.float32)
+    got, ref = run_gemm(ta, tb, m, n, k, a, b, F16, F16, c_dt, hip.GEMM_F16, alpha=0.5, bias=bias, c0=c0)
+    assert_close(got, ref, 2e-2, "two wave groups")
+    if c_dt == F32:
+        assert np.sqrt(np.mean((got - ref) ** 2)) < 1e-5 * np.sqrt(np.mean(ref ** 2)) * np.sqrt(k)
+        ai = rng.integers(-8, 9, a.shape).astype(np.float32)
+        bi = rng.integers(-4, 5, b.shape).astype(np.float32)
+        got, ref = run_gemm(ta, tb, m, n, k, ai, bi, F16, F16, F32, hip.GEMM_F16)
+        assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("ta,tb", [(0, 1), (0, 0), (1, 0), (1, 1)])
 @pytest.mark.parametrize("a_dt,b_dt", [(F32, F16), (F16, F32), (F32, F32)])
 def test_gemm_staged_matches_plain_entry(ta, tb, a_dt, b_dt):
     rng = np.random.default_rng(8)
@@ -373,7 +396,8 @@ def test_gemm_rejects_bad_arguments():
 
 
 @pytest.mark.parametrize("dtype", [F16, BF16])
-@pytest.mark.parametrize("rows,out,inn", [(512, 1024, 256), (200, 520, 96), (2048, 4096, 1024), (2048, 12288, 1024)])
+@pytest.mark.parametrize("rows,out,inn", [(512, 1024, 256), (200, 520, 96), (2048, 4096, 1024), (2048, 12288, 1024),
+                                          (512, 16384, 2048)])   # the last: 256 x 128 tiles on two groups of waves
 def test_linear_gelu_epilogue_writes_both_tensors(dtype, rows, out, inn):
     """br_hip_linear_gelu: u = x.W^T + bias and y = gelu(u) from one product.
     u against the fp64 product of the stored operands, y against the oracle's
